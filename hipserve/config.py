@@ -383,8 +383,8 @@ def resolve_model_config(model: str, name: str | None = None) -> ModelConfig:
         return PRESETS[k]
     if os.path.isdir(model) and os.path.exists(os.path.join(model, "config.json")):
         with open(os.path.join(model, "config.json")) as f:
-            return _with_preprocessor(ModelConfig.from_hf_dict(json.load(f), name=name or os.path.basename(model)),
-                                      model)
+            cfg = config_from_dict(json.load(f), name=name or os.path.basename(os.path.normpath(model)))
+            return _with_preprocessor(cfg, model) if isinstance(cfg, ModelConfig) else cfg
     if model.endswith(".gguf") and os.path.exists(model):
         from .weights.gguf import GGUFFile
 
@@ -551,3 +551,177 @@ class EngineConfig:
     @property
     def model_name(self) -> str:
         return self.served_model_name or self.model
+
+
+# ---------------------------------------------------------------------------------
+# Layer-list ("hybrid") decoders: the config file lists the layers one by one, each
+# with its sequence mixer and its feed-forward, instead of one repeated block.
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention through low-rank latents: queries go through a ``q_rank`` latent, keys
+    and values are expanded per head from one ``kv_rank`` latent per token, and a
+    ``rot_dim`` rotary key part is shared by all heads. Only the latent and the rotary
+    key part are cached. ``window`` 0 = plain causal attention."""
+    heads: int
+    dim: int            # unrotated query/key dims per head
+    rot_dim: int        # rotated query/key dims per head (one shared key part)
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    window: int = 0
+    rot_base: float = 10000.0
+    rot_dims: int = 0   # leading dims of the rotated part that are rotated (0 = all of rot_dim)
+
+    kind = "latent_attention"
+
+    @property
+    def key_dim(self) -> int:
+        """Cached elements per token."""
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass(frozen=True)
+class MinGRUSpec:
+    """Gated linear recurrence whose gates read only the current token (minGRU)."""
+    width: int
+
+    kind = "mingru"
+
+
+@dataclass(frozen=True)
+class TableMoESpec:
+    """Mixture of small feed-forwards whose experts are looked up per token id in a
+    table (no learned router at run time); every chosen expert weighs 1 / top."""
+    experts: int
+    top: int
+    ff: int
+
+    kind = "moe"
+
+
+@dataclass(frozen=True)
+class HybridLayerSpec:
+    mixer: object               # LatentAttentionSpec | MinGRUSpec
+    mlp: object | None          # TableMoESpec | None
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    """A decoder given as a list of layers (``layers[i]``), of which the span
+    ``loop_start .. loop_stop - 1`` runs ``loop_times`` times in a row with the same
+    weights. Carries the attributes the engine reads from any model config."""
+    name: str = "hybrid"
+    architecture: str = "kesirax"
+    family: str = "kesirax"
+    hidden_size: int = 256
+    vocab_size: int = 512
+    layers: tuple = ()
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    norm_eps: float = 1e-6
+    norm_groups: int = 1
+    logit_scale: float = 1.0
+    max_position_embeddings: int = 1 << 20   # rotary angles are computed, not tabulated
+    bos_token_id: int | None = None
+    eos_token_id: tuple = ()
+    vision: object = None
+    num_experts: int = 0                      # no learned-router MoE (engine start-up tuning keys on it)
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list:
+        """Layer runs in execution order: (layer index, pass index, starts_pass) where
+        ``starts_pass`` marks the first layer of every pass of the loop but the first."""
+        a, b, n = self.loop_start, self.loop_stop, self.loop_times
+        out = [(i, 0, False) for i in range(0, a)]
+        for t in range(n if b > a else 0):
+            out += [(i, t, t > 0 and i == a) for i in range(a, b)]
+        out += [(i, 0, False) for i in range(b if b > a else a, len(self.layers))]
+        return out
+
+    def num_params(self) -> int:
+        H, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            m = l.mixer
+            if isinstance(m, LatentAttentionSpec):
+                n += H * (m.q_rank + m.key_dim + m.heads) + m.q_rank * m.heads * (m.dim + m.rot_dim)
+                n += m.kv_rank * m.heads * (m.dim + m.vdim) + m.heads * m.vdim * H
+            else:
+                n += 4 * H * m.width
+            if l.mlp is not None:
+                n += 2 * l.mlp.experts * l.mlp.ff * H
+        return n
+
+    def replace(self, **kw) -> "HybridConfig":
+        return dataclasses.replace(self, **kw)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "model") -> "HybridConfig":
+        layers = []
+        for l in d["layers"]:
+            m = l["mixer"]
+            if l["type"] == "latent_attention":
+                rot = m.get("rot") or {}
+                mixer = LatentAttentionSpec(
+                    heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                    q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                    window=int((m.get("mask") or {}).get("size") or 0),
+                    rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims") or m["rot_dim"]))
+            elif l["type"] == "mingru":
+                mixer = MinGRUSpec(width=int(m["width"]))
+            else:
+                raise NotImplementedError(f"unknown mixer {l['type']!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") != "moe":
+                    raise NotImplementedError(f"unknown feed-forward {f.get('kind')!r}")
+                mlp = TableMoESpec(experts=int(f["router"]["experts"]), top=int(f["router"]["top"]),
+                                   ff=int(f["expert"]["ff"]))
+            layers.append(HybridLayerSpec(mixer, mlp))
+        lp = d.get("loop") or {}
+        norm = d.get("norm") or {}
+        eos = d.get("eos_token_id", ())
+        eos = tuple(eos) if isinstance(eos, (list, tuple)) else (eos,)
+        return HybridConfig(
+            name=name, hidden_size=int(d["width"]), vocab_size=int(d["vocab"]), layers=tuple(layers),
+            loop_start=int(lp.get("start", 0)), loop_stop=int(lp.get("stop", 0)), loop_times=int(lp.get("times", 1)),
+            norm_eps=float(norm.get("eps", 1e-6)), norm_groups=int(norm.get("groups", 1)),
+            logit_scale=float(d.get("logit_scale", 1.0)), bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
+
+
+def config_from_dict(d: dict, name: str = "model"):
+    """Model config of a ``config.json``: the layer-list designs are recognised by their
+    ``architecture`` key, everything else is a HuggingFace config."""
+    if str(d.get("architecture", "")).lower() == "kesirax":
+        return HybridConfig.from_dict(d, name=name)
+    return ModelConfig.from_hf_dict(d, name=name)
+
+
+def _mini_kesirax(name, H, V, attn, gru, ff, order, loop=(0, 0, 1), groups=1):
+    a = LatentAttentionSpec(**attn)
+    g = MinGRUSpec(gru)
+    f = TableMoESpec(**ff) if ff else None
+    return HybridConfig(name=name, hidden_size=H, vocab_size=V,
+                        layers=tuple(HybridLayerSpec(a if c == "a" else g, f) for c in order),
+                        loop_start=loop[0], loop_stop=loop[1], loop_times=loop[2], norm_groups=groups,
+                        eos_token_id=(2,), bos_token_id=1)
+
+
+PRESETS.update({
+    # CPU plumbing size
+    "tiny-kesirax": _mini_kesirax("tiny-kesirax", 64, 320,
+                                  dict(heads=3, dim=16, rot_dim=8, vdim=24, q_rank=40, kv_rank=32, scale=24 ** -0.5,
+                                       window=24, rot_base=10000.0),
+                                  48, dict(experts=4, top=2, ff=40), "gaag", loop=(1, 3, 2), groups=4),
+    # GPU-test size
+    "small-kesirax": _mini_kesirax("small-kesirax", 512, 1024,
+                                   dict(heads=8, dim=64, rot_dim=32, vdim=64, q_rank=192, kv_rank=128,
+                                        scale=96 ** -0.5, window=160, rot_base=50000.0),
+                                   768, dict(experts=8, top=2, ff=256), "agag", loop=(0, 2, 2), groups=2),
+})

@@ -22,6 +22,7 @@ from .metrics import EngineMetrics
 from .model_runner import ModelRunner
 from .request import RequestOutput, SamplingParams, Sequence, Status
 from .scheduler import ScheduledSeq, Scheduler, SchedulerOutput
+from .state_manager import StateSlots
 
 PLACEHOLDER = -1  # output token whose value is still on the GPU (decode lookahead)
 
@@ -58,9 +59,13 @@ class LLMEngine:
         cfg = self.cfg
         self.runner = ModelRunner(cfg, self.model_cfg, self.tp)
         self.max_model_len = self.runner.max_model_len
-        self.blocks = BlockManager(self.runner.usable_blocks, cfg.block_size, cfg.enable_prefix_caching)
+        # recurrent layers keep their state per sequence, not per block: a cached prefix
+        # cannot be resumed from, so such models run without the prefix cache
+        self.states = StateSlots(self.runner.num_state_slots) if self.runner.needs_state else None
+        self.blocks = BlockManager(self.runner.usable_blocks, cfg.block_size,
+                                   cfg.enable_prefix_caching and self.states is None)
         self.scheduler = Scheduler(self.blocks, cfg.max_num_seqs, cfg.max_num_batched_tokens,
-                                   self.max_model_len)
+                                   self.max_model_len, states=self.states)
         self.seqs: dict[str, Sequence] = {}
         self.detok: dict[str, IncrementalDetokenizer] = {}
         self._ids = itertools.count()

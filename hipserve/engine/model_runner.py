@@ -21,7 +21,8 @@ import numpy as np
 import torch
 
 from ..config import EngineConfig, ModelConfig
-from ..models.llama import AttnMeta, LlamaModel
+from ..models.llama import AttnMeta
+from ..models.registry import build_model, load_weights, model_class
 from ..ops import get_ops
 from ..parallel.comm import TPGroup
 from ..runtime import native
@@ -61,6 +62,12 @@ class StepInputs:
     # decode lookahead: per decode row, the row of the PREVIOUS graph step's sampled
     # tokens that is this row's input id (-1: use ids[row]); consumed on the device
     src: np.ndarray | None = None
+    # per-sequence view of the step (prefill sequences, then decode ones) for the mixers that index
+    # it by sequence: row offsets int32 [n+1], context lengths [n], block tables [n, W], state slots [n]
+    seq_cu: np.ndarray | None = None
+    seq_ctx: np.ndarray | None = None
+    seq_bt: np.ndarray | None = None
+    seq_state: np.ndarray | None = None
     extra: dict = field(default_factory=dict)
 
 
@@ -92,13 +99,16 @@ class ModelRunner:
             torch.cuda.set_device(self.device)
         self.dtype = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "auto": torch.bfloat16,
                       "float32": torch.float32, "fp32": torch.float32}[ecfg.dtype]
-        if self.device.type == "cuda" and self.dtype != torch.bfloat16:
-            raise ValueError("the gfx950 kernels run bf16 activations; use --dtype bfloat16")
+        if (self.device.type == "cuda" and self.dtype != torch.bfloat16
+                and not getattr(model_class(mcfg), "supports_fp32", False)):
+            raise ValueError("the gfx950 kernels of this model run bf16 activations; use --dtype bfloat16")
         self.ops = get_ops(self.device)
         self.max_model_len = min(ecfg.max_model_len or mcfg.max_position_embeddings,
                                  mcfg.max_position_embeddings)
         self.block_size = ecfg.block_size
-        self.model = LlamaModel(mcfg, tp, self.device, self.dtype, self.ops, max_pos=self.max_model_len)
+        self.model = build_model(mcfg, tp, self.device, self.dtype, self.ops, max_pos=self.max_model_len)
+        # dense-transformer start-up tuning (decode GEMM autotune, weight packing, prefill padding)
+        self.dense_tuning = hasattr(self.model, "gemm_shapes")
         self.model.decode_partition = ecfg.decode_partition
         self.model.block_size_hint = ecfg.block_size
         if ecfg.kv_fp8:  # e4m3 paged KV cache (the fused qkv -> attention kernel writes bf16 only)
@@ -137,7 +147,7 @@ class ModelRunner:
         # copies need scratch, and weights whose winner is the packed decode GEMM get
         # their pre-shuffled copy (gemm.PACKED) allocated before the pool is sized
         self.gemm_report = []
-        if self.device.type == "cuda" and ecfg.extra.get("gemm_autotune", True):
+        if self.device.type == "cuda" and self.dense_tuning and ecfg.extra.get("gemm_autotune", True):
             from ..ops import gemm
 
             ms = [b for b in self.buckets if b <= 64]
@@ -201,7 +211,7 @@ class ModelRunner:
         # prefill GEMMs per 256-row count once and pads a chunk to the fastest count at
         # or above it (padding rows: token 0, no KV write, outputs unused)
         self.prefill_pad = None
-        if self.device.type == "cuda" and ecfg.extra.get("prefill_pad", True) and tp.rank == 0:
+        if self.device.type == "cuda" and self.dense_tuning and ecfg.extra.get("prefill_pad", True) and tp.rank == 0:
             self.prefill_pad = self._probe_prefill_pad()
         # device penalty state: one slot per concurrently running sequence (a slot is
         # held from the first sample to finish / abort / preemption), so a slot is
@@ -216,21 +226,30 @@ class ModelRunner:
         t1 = time.time()
         self.num_blocks = self._num_kv_blocks()
         self.kv = self.model.allocate_kv_cache(self.num_blocks, self.block_size)
+        # recurrent layers: one state slot per running sequence, plus a scratch slot for padding rows
+        self.needs_state = bool(getattr(self.model, "needs_state", False))
+        self.num_state_slots = max(1, ecfg.max_num_seqs) if self.needs_state else 0
+        self.state = self.model.allocate_state(self.num_state_slots + 1) if self.needs_state else None
+        # models whose mixers index the step by sequence (row offsets, lengths, block tables, state slots)
+        self.seq_meta = hasattr(self.model, "runs")
         self.init_times["kv_alloc_s"] = round(time.time() - t1, 2)
         self.pad_block = self.num_blocks - 1          # scratch block for graph padding rows
         self.width = -(-self.max_model_len // self.block_size)
         part = ecfg.decode_partition
         self.max_parts = -(-self.width * self.block_size // part)
-        nq = self.model.nq
-        self.tmp_out = torch.empty(self.max_bs, nq, self.max_parts, mcfg.head_dim,
-                                   device=self.device, dtype=torch.float32)
-        self.tmp_ml = torch.empty(self.max_bs, nq, self.max_parts, 2, device=self.device,
-                                  dtype=torch.float32)
+        self.tmp_out = self.tmp_ml = None
+        if hasattr(self.model, "nq"):  # split-context decode attention workspace
+            nq = self.model.nq
+            self.tmp_out = torch.empty(self.max_bs, nq, self.max_parts, mcfg.head_dim,
+                                       device=self.device, dtype=torch.float32)
+            self.tmp_ml = torch.empty(self.max_bs, nq, self.max_parts, 2, device=self.device,
+                                      dtype=torch.float32)
         self.stats = {"graph_steps": 0, "eager_steps": 0}  # which path each step took
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.graph_pool = None
         self._static = None
-        self.use_graphs = self.device.type == "cuda" and not ecfg.enforce_eager
+        self.use_graphs = (self.device.type == "cuda" and not ecfg.enforce_eager
+                           and getattr(self.model, "graph_decode", True))
         if self.use_graphs:
             self._capture_graphs()
         self.init_times["graph_capture_s"] = round(getattr(self, "graph_capture_time", 0.0), 2)
@@ -257,9 +276,7 @@ class ModelRunner:
         elif fmt == "dummy":
             self.model.allocate_random(seed=self.ecfg.seed)
         elif fmt == "safetensors":
-            from ..weights.safetensors_loader import load_hf_weights
-
-            load_hf_weights(self.model, model)
+            load_weights(self.model, model)
         elif fmt == "gguf":
             from ..weights.gguf import load_gguf_weights
 
@@ -328,8 +345,14 @@ class ModelRunner:
         torch.cuda.synchronize(self.device)
         free, total = torch.cuda.mem_get_info(self.device)
         used = total - free
-        H, I = self.mcfg.hidden_size, self.model.inter
         T = self.ecfg.max_num_batched_tokens
+        if hasattr(self.model, "step_workspace_bytes"):
+            reserve = self.model.step_workspace_bytes(T, self.ecfg.max_num_seqs) + (2 << 30)
+            n = int((total * self.ecfg.gpu_memory_utilization - used - reserve) // per_block)
+            if n < 16:
+                raise RuntimeError("not enough GPU memory for the cache")
+            return self.tp.min_int(n)
+        H, I = self.mcfg.hidden_size, self.model.inter
         qkv = (self.model.nq + 2 * self.model.nkv) * self.mcfg.head_dim
         act = T * (2 * I + I + qkv + 6 * H) * 2 * 2
         logits = self.ecfg.max_num_seqs * self.mcfg.vocab_size * 4 * 3
@@ -502,6 +525,16 @@ class ModelRunner:
         inp = StepInputs(ids, pos, slots, Tp, len(so.decode), bt_p, cu_q, ctx_p, tiles, bt_d, ctx_d,
                          np.array(rows, dtype=np.int64), temp, topk, topp, seeds, steps,
                          pen_slot, pen_vals, nlp, pen_init, topn)
+        if self.seq_meta:
+            cu = np.zeros(len(seqs) + 1, dtype=np.int32)
+            cu[1:] = np.cumsum([s.num_tokens for s in seqs])
+            inp.seq_cu = cu
+            inp.seq_ctx = np.array(ends, dtype=np.int32)
+            inp.seq_bt = bt
+            if self.needs_state:
+                inp.seq_state = np.array([s.seq.state_slot for s in seqs], dtype=np.int32)
+        if so.logits_rows is not None:  # teacher-forced replay: logits at the asked rows, nothing sampled
+            inp.logits_rows = np.asarray(so.logits_rows, dtype=np.int64)
         if any(s.seq.mm is not None for s in seqs):
             self._prepare_mm(seqs, inp)
         return inp
@@ -568,10 +601,12 @@ class ModelRunner:
                 and 0 < inp.num_decode <= self.buckets[-1])
 
     @torch.inference_mode()
-    def execute(self, inp: StepInputs):
-        """Returns (tokens np.int64 [n], logprobs np.float32 [n], top_logprobs or None)."""
+    def execute(self, inp: StepInputs, return_logits: bool = False):
+        """Returns (tokens np.int64 [n], logprobs np.float32 [n], top_logprobs or None);
+        with ``return_logits`` the fp32 logits [n, vocab] of the step's logits rows instead
+        (nothing is sampled)."""
         n = len(inp.logits_rows)
-        if self.graph_eligible(inp):
+        if self.graph_eligible(inp) and not return_logits:
             return self.wait(self.launch(inp))
         if inp.src is not None:
             raise RuntimeError("device-side input ids (lookahead) need the hipGraph decode path")
@@ -587,13 +622,22 @@ class ModelRunner:
         if inp.num_decode > self.max_bs:
             meta.tmp_out = torch.empty(inp.num_decode, *self.tmp_out.shape[1:], device=self.device)
             meta.tmp_ml = torch.empty(inp.num_decode, *self.tmp_ml.shape[1:], device=self.device)
+        if inp.seq_cu is not None:
+            meta.seq_cu, meta.seq_ctx = self._t(inp.seq_cu), self._t(inp.seq_ctx)
+            meta.seq_bt, meta.seq_state = self._t(inp.seq_bt), self._t(inp.seq_state)
+            meta.state = self.state
+            meta.max_q = int(np.max(np.diff(inp.seq_cu))) if len(inp.seq_cu) > 1 else 0
         if "mm" in inp.extra:
             self._attach_mm(inp.extra["mm"], meta, len(inp.ids))
         hidden = self.model.forward(ids, meta, self.kv)
         if n == 0:
+            if return_logits:
+                return np.zeros((0, self.mcfg.vocab_size), np.float32)
             return np.zeros(0, np.int64), np.zeros(0, np.float32), None
         rows = self._t(inp.logits_rows)
         logits = self.model.compute_logits(hidden.index_select(0, rows))
+        if return_logits:
+            return logits.float().cpu().numpy()
         top = None
         if inp.top_logprobs:  # raw (pre-penalty) log-probs, as vLLM's default mode
             ti = torch.empty(n, TOP_LOGPROBS, dtype=torch.int32, device=self.device)

@@ -38,6 +38,8 @@ class SchedulerOutput:
     prefill: list[ScheduledSeq] = field(default_factory=list)
     decode: list[ScheduledSeq] = field(default_factory=list)
     preempted: list[Sequence] = field(default_factory=list)
+    # teacher-forced replay (engine/trace.py): batch rows whose logits are wanted instead of sampling
+    logits_rows: list | None = None
 
     @property
     def num_tokens(self) -> int:
@@ -50,8 +52,9 @@ class SchedulerOutput:
 
 class Scheduler:
     def __init__(self, blocks: BlockManager, max_num_seqs: int, max_num_batched_tokens: int,
-                 max_model_len: int):
+                 max_model_len: int, states=None):
         self.blocks = blocks
+        self.states = states  # engine/state_manager.py StateSlots of a model with recurrent layers, else None
         self.max_num_seqs = max_num_seqs
         self.max_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len
@@ -68,11 +71,17 @@ class Scheduler:
             for s in list(q):
                 if s.request_id == request_id:
                     q.remove(s)
-                    self.blocks.free(s)
+                    self._release(s)
                     s.status = Status.FINISHED
                     s.finish_reason = "abort"
                     return s
         return None
+
+    def _release(self, seq: Sequence):
+        """Cache blocks and the state slot of a sequence that leaves the running set."""
+        self.blocks.free(seq)
+        if self.states is not None:
+            self.states.free(seq)
 
     def has_unfinished(self) -> bool:
         return bool(self.waiting or self.running)
@@ -87,7 +96,7 @@ class Scheduler:
 
     def _preempt(self, seq: Sequence, out: SchedulerOutput):
         self.running.remove(seq)
-        self.blocks.free(seq)
+        self._release(seq)
         seq.num_computed_tokens = 0
         seq.status = Status.PREEMPTED
         self.waiting.appendleft(seq)
@@ -122,6 +131,8 @@ class Scheduler:
         if not out.preempted:
             while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
                 seq = self.waiting[0]
+                if self.states is not None and not self.states.can_allocate(seq):
+                    break  # every state slot is held by a running sequence
                 if seq.num_computed_tokens == 0 and not seq.block_ids:
                     self.blocks.match_prefix(seq)
                 n = min(seq.num_uncomputed, budget)
@@ -135,7 +146,7 @@ class Scheduler:
                         # nothing else can free memory: the request can never fit
                         if not self.blocks.can_grow(seq, target):
                             self.waiting.popleft()
-                            self.blocks.free(seq)
+                            self._release(seq)
                             seq.status = Status.FINISHED
                             seq.finish_reason = "length"
                             out.preempted.append(seq)
@@ -145,6 +156,8 @@ class Scheduler:
                     break
                 self.waiting.popleft()
                 self.blocks.grow(seq, target)
+                if self.states is not None:
+                    self.states.allocate(seq)
                 seq.status = Status.RUNNING
                 self.running.append(seq)
                 out.prefill.append(ScheduledSeq(seq, seq.num_computed_tokens, target))
@@ -156,4 +169,4 @@ class Scheduler:
         seq.finish_reason = reason
         if seq in self.running:
             self.running.remove(seq)
-        self.blocks.free(seq)
+        self._release(seq)

@@ -66,6 +66,15 @@ class AttnMeta:
     # decode lookahead (model_runner): (src, tok) — row i's input id is tok[src[i]]
     # where src[i] >= 0 (the previous graph step's sampled id), else ids[i]
     id_src: tuple | None = None
+    # per-sequence view of the step (prefill sequences, then decode ones) for the layer-list
+    # decoders' mixers: row offsets int32 [n+1], context lengths after the step [n], block tables
+    # [n, W], recurrent-state slots [n], the state tensors per layer run, longest row count (host)
+    seq_cu: torch.Tensor | None = None
+    seq_ctx: torch.Tensor | None = None
+    seq_bt: torch.Tensor | None = None
+    seq_state: torch.Tensor | None = None
+    state: list | None = None
+    max_q: int = 0
 
 
 @dataclass

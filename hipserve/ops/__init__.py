@@ -224,6 +224,30 @@ class ReferenceOps:
         out.copy_(ref.vision_attention(qkv, cu_seqlens, nh, D, scale))
         return out
 
+    # ---- layer-list decoders (models/mixers.py)
+    def scaled_add_group_rmsnorm(self, out, residual, w, groups, eps, mix=None, ls1=None, y=None, pair_slot=None,
+                                 top=0, ls2=None, extra=None):
+        ref.scaled_add_group_rmsnorm(out, residual, w, groups, eps, mix, ls1, y, pair_slot, top, ls2, extra)
+        return out
+
+    def latent_prepare(self, cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
+                       rot_dim, eps):
+        ref.latent_prepare(cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank, rot_dim, eps)
+
+    def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
+                         gate_off, scale, window):
+        ref.latent_attention(o_lat, q_abs, q, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, inv_freq,
+                             heads, dim, rot_dim, kv_rank, gate_off, scale, window)
+
+    def mingru_scan(self, y, state, proj, b_z, b_x, meta):
+        ref.mingru_scan(y, state, proj, b_z, b_x, meta.seq_cu, meta.seq_ctx, meta.seq_state)
+
+    def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
+        ref.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
+
+    def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
+        ref.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
+
     def sample(self, out_tok, out_lp, logits, temperature, top_k, top_p, seeds, steps, two_rounds=True):
         t, lp = ref.sample(logits, temperature, top_k, top_p, seeds, steps, bf16_row=False)
         n = t.shape[0]

@@ -393,3 +393,139 @@ def top_logprobs(logits, nreq, out_ids, out_lp):
         for i, v in enumerate(order):
             out_ids[r, i] = v
             out_lp[r, i] = ls[v]
+
+
+# ---------------------------------------------------------------------------------
+# layer-list decoders (models/mixers.py): grouped norm + residual update, latent
+# attention on a paged latent cache, minGRU scan over state slots, table-routed experts
+
+def scaled_add_group_rmsnorm(out, residual, w, groups, eps, mix=None, ls1=None, y=None, pair_slot=None, top=0,
+                             ls2=None, extra=None):
+    """residual (fp32, in place) += ls1 * mix + ls2 * mean_j y[pair_slot[t * top + j]] + extra;
+    out = residual normalised in ``groups`` equal consecutive parts, times w."""
+    T, H = residual.shape
+    if mix is not None:
+        residual += mix.float() * ls1.float()
+    if y is not None:
+        rows = y.float().index_select(0, pair_slot.long()).view(T, top, H)
+        residual += rows.sum(1) * (1.0 / top) * ls2.float()
+    if extra is not None:
+        residual += extra.float()
+    g = residual.view(T, groups, H // groups)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+    out.copy_((g.reshape(T, H) * w.float()).to(out.dtype))
+
+
+def partial_rope(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """Rotate-half RoPE of the first 2 * len(inv_freq) elements of the last dim (fp32);
+    pair (i, i + n): (u cos a - v sin a, v cos a + u sin a), a = pos * inv_freq[i]."""
+    n = inv_freq.shape[0]
+    a = pos.float().unsqueeze(-1) * inv_freq.float()
+    while a.dim() < x.dim():
+        a = a.unsqueeze(-2)
+    c, s = a.cos(), a.sin()
+    u, v = x[..., :n].float(), x[..., n:2 * n].float()
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * n:].float()], -1)
+
+
+def latent_prepare(cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank, rot_dim, eps):
+    """proj rows = [q latent | kv latent | rotary key | ...]: cq = RMSNorm(q latent) * q_norm;
+    cache[slot] = [RMSNorm(kv latent) * kv_norm | RoPE(rotary key)] for slots >= 0."""
+    p = proj.float()
+    a = p[:, :q_rank]
+    cq.copy_((a * torch.rsqrt(a.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()).to(cq.dtype))
+    c = p[:, q_rank:q_rank + kv_rank]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kv_norm.float()
+    kr = partial_rope(p[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim], positions, inv_freq)
+    row = torch.cat([c, kr], -1).to(cache.dtype)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok]] = row[ok]
+
+
+def latent_attention(o_lat, q_abs, q, proj, cache, seq_cu, seq_ctx, seq_bt, inv_freq, heads, dim, rot_dim,
+                     kv_rank, gate_off, scale, window):
+    """Per sequence s with rows cu[s]..cu[s+1]-1 at positions ctx[s] - n .. ctx[s] - 1: scores of
+    head h = (q_abs[h, t] . latent + RoPE(q[t, h, dim:]) . rotary key) * scale over the keys
+    0 <= pos - j < window (window 0: all j <= pos), softmax, latent-space output times
+    sigmoid(proj[t, gate_off + h])."""
+    bs = cache.shape[1]
+    flat = cache.view(-1, cache.shape[-1])
+    cu = [int(v) for v in seq_cu]
+    T = q.shape[0]
+    qh = q.view(T, heads, dim + rot_dim)
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if a == b:
+            continue
+        ctx = int(seq_ctx[s])
+        pos = torch.arange(ctx - (b - a), ctx, device=q.device)
+        lo = 0 if window <= 0 else max(0, int(pos[0]) - window + 1)
+        j = torch.arange(lo, ctx, device=q.device)
+        rows = seq_bt[s].long()[j // bs] * bs + j % bs
+        kv = flat[rows].float()                                  # [n_keys, kv_rank + rot_dim]
+        qr = partial_rope(qh[a:b, :, dim:], pos, inv_freq)       # [n, heads, rot_dim]
+        sc = torch.einsum("hnk,jk->hnj", q_abs[:, a:b].float(), kv[:, :kv_rank])
+        sc = (sc + torch.einsum("nhr,jr->hnj", qr, kv[:, kv_rank:])) * scale
+        d = pos[:, None] - j[None]
+        ok = (d >= 0) & ((d < window) if window > 0 else (d >= 0))
+        sc = sc.masked_fill(~ok, float("-inf"))
+        o = torch.einsum("hnj,jk->hnk", torch.softmax(sc, -1), kv[:, :kv_rank])
+        g = torch.sigmoid(proj[a:b, gate_off:gate_off + heads].float())   # [n, heads]
+        o_lat[:, a:b] = (o * g.t().unsqueeze(-1)).to(o_lat.dtype)
+
+
+def mingru_scan(y, state, proj, b_z, b_x, seq_cu, seq_ctx, seq_state):
+    """proj rows = [z | x | g] pre-activations. Per sequence, from its state slot (zero when
+    the step starts at position 0): S = (1 - z) S + z c, z = sigmoid(. + b_z), u = . + b_x,
+    c = u + 0.5 (u >= 0) or sigmoid(u); y = S * silu(g). The slot gets the last S."""
+    n = state.shape[1]
+    cu = [int(v) for v in seq_cu]
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if a == b:
+            continue
+        slot = int(seq_state[s])
+        S = state[slot].clone() if int(seq_ctx[s]) - (b - a) > 0 else torch.zeros_like(state[slot])
+        p = proj[a:b].float()
+        z = torch.sigmoid(p[:, :n] + b_z)
+        u = p[:, n:2 * n] + b_x
+        c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        g = p[:, 2 * n:]
+        g = g * torch.sigmoid(g)
+        for t in range(b - a):
+            S = (1 - z[t]) * S + z[t] * c[t]
+            y[a + t] = (S * g[t]).to(y.dtype)
+        state[slot] = S
+
+
+def moe_align(experts, E, tile, slots, tile_expert, pair_slot):
+    """Pairs sorted by expert into tiles of ``tile`` slots: slots[pos] = pair index or -1
+    (padding), tile_expert[t] = the tile's expert or -1, pair_slot[p] = the pair's slot."""
+    slots.fill_(-1)
+    tile_expert.fill_(-1)
+    pos = 0
+    ex = experts.tolist()
+    for e in range(E):
+        ps = [p for p, v in enumerate(ex) if v == e]
+        for k, p in enumerate(ps):
+            slots[pos + k] = p
+            pair_slot[p] = pos + k
+        nt = -(-len(ps) // tile)
+        tile_expert[pos // tile:pos // tile + nt] = e
+        pos += nt * tile
+
+
+def expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2):
+    """out[slot] = act(W[e(slot)] . x[row(slot)]); row = slots[slot] // gather_k (gather_k > 0)
+    or the slot itself; act = squared ReLU or none. Padding slots are left untouched."""
+    sl = slots.tolist()
+    te = tile_expert.tolist()
+    for s, p in enumerate(sl):
+        if p < 0:
+            continue
+        e = te[s // tile]
+        row = p // gather_k if gather_k > 0 else s
+        v = w[e].float() @ x[row].float()
+        if relu2:
+            v = torch.relu(v) ** 2
+        out[s] = v.to(out.dtype)

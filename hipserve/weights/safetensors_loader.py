@@ -468,3 +468,17 @@ def random_hf_tensors(cfg, seed: int = 0, std: float = 0.05) -> dict[str, torch.
             t[p + "mlp.up_proj.weight"] = rnd(I, H)
             t[p + "mlp.down_proj.weight"] = rnd(H, I)
     return t
+
+
+def load_named_tensors(model, model_path: str):
+    """Checkpoints whose tensor names are the model's own (the layer-list decoders):
+    every tensor is handed to ``model.load_tensors`` by name, read lazily from the
+    safetensors shards. Unknown names in the file are ignored, missing ones raise."""
+    ck = _Ckpt(resolve_checkpoint_dir(model_path))
+
+    def get(name: str) -> torch.Tensor:
+        if not ck.has(name):
+            raise KeyError(f"{model_path}: tensor {name!r} is not in the checkpoint")
+        return ck.full(name)
+
+    model.load_tensors(get)
