@@ -1,0 +1,42 @@
+// Launchers of the layer-list decoders' kernels (csrc/kernels/seq/*.hip): grouped RMSNorm
+// fused with the scaled residual update, latent attention on a paged latent cache, the
+// minGRU scan over state slots, and the table-routed experts' GEMMs. Every launcher has a
+// bf16 and a true fp32 build (``f32``): the activations' element type; norms, scores,
+// softmax, recurrences and the residual stream are fp32 in both.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace hipserve {
+
+// residual[T, H] (fp32, in place) += ls1 * mix + ls2 * (1/top) * sum_j y[pair_slot[t*top+j]] + extra;
+// out = residual normalised in `groups` consecutive parts, times w (fp32 [H]). Null inputs are skipped.
+void launch_scaled_add_group_rmsnorm(void* out, float* residual, const float* w, int T, int H, int groups, float eps,
+                                     const void* mix, const float* ls1, const void* y, const int* pair_slot, int top,
+                                     const float* ls2, const void* extra, bool f32, hipStream_t s);
+
+// proj[T, ld] rows = [q latent (q_rank) | kv latent (kv_rank) | rotary key (rot_dim) | ...]:
+// cq[T, q_rank] = RMSNorm(q latent) * q_norm; cache row slots[t] (>= 0) = [RMSNorm(kv latent) * kv_norm |
+// RoPE(rotary key)], rotate-half over the first 2 * nfreq dims with angle pos * inv_freq[i].
+void launch_latent_prepare(void* cq, void* cache, const void* proj, long ld, const long* positions, const long* slots,
+                           const float* q_norm, const float* kv_norm, const float* inv_freq, int nfreq, int T,
+                           int q_rank, int kv_rank, int rot_dim, float eps, bool f32, hipStream_t s);
+
+// Attention of every (token, head) row on the cached latents of its sequence; sequences
+// seq0 .. seq1-1 of the step, `tq` tokens per workgroup. o_lat[heads, T, kv_rank] gets the
+// latent-space output times sigmoid(proj[t, gate_off + h]).
+void launch_latent_attention(void* o_lat, const float* q_abs, const void* q, const void* proj, long proj_ld,
+                             const void* cache, int block_size, const int* seq_cu, const int* seq_ctx,
+                             const int* seq_bt, int bt_width, int seq0, int seq1, int rows_bound, int tq,
+                             const float* inv_freq, int nfreq, int T, int heads, int dim, int rot_dim, int kv_rank,
+                             int gate_off, float scale, int window, bool f32, hipStream_t s);
+
+// minGRU over the step's rows of every sequence, from / to its fp32 state slot.
+void launch_mingru_scan(void* y, float* state, const void* proj, const float* b_z, const float* b_x,
+                        const int* seq_cu, const int* seq_ctx, const int* seq_state, int nseq, int width, int max_q,
+                        bool f32, hipStream_t s);
+
+// out[slot, N] = act(W[e(tile)] [N, K] . x[row(slot)]) over moe_align tiles of `tile` slots.
+void launch_expert_gemm(void* out, const void* x, long x_ld, const void* w, const int* slots, const int* tile_expert,
+                        int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, bool f32, hipStream_t s);
+
+}  // namespace hipserve

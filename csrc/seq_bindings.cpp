@@ -1,0 +1,178 @@
+// torch.ops.hipserve_seq.* — the layer-list decoders' kernels (csrc/kernels/seq/*.hip), built as
+// their own library (hipserve/_C_seq.so) so a model of these designs compiles only what it runs.
+// All ops write into caller-provided outputs (no allocation except moe_align's scratch, no host sync).
+#include <torch/library.h>
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+
+#include "hipserve/kernels.h"
+#include "hipserve/seq_kernels.h"
+
+namespace {
+
+hipStream_t cur_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+#define CHECK_DEV(x) TORCH_CHECK((x).is_cuda(), #x " must be a GPU tensor")
+#define CHECK_CONTIG(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous")
+#define CHECK_F32(x) TORCH_CHECK((x).scalar_type() == at::kFloat && (x).is_contiguous(), #x " must be contiguous fp32")
+#define CHECK_I32(x) TORCH_CHECK((x).scalar_type() == at::kInt && (x).is_contiguous(), #x " must be contiguous int32")
+
+bool is_f32(const at::Tensor& t, const char* who) {
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, who, ": bf16 or fp32 activations");
+  return t.scalar_type() == at::kFloat;
+}
+
+const void* opt_ptr(const c10::optional<at::Tensor>& t) { return t.has_value() ? t->data_ptr() : nullptr; }
+
+void scaled_add_group_rmsnorm(at::Tensor& out, at::Tensor& residual, const at::Tensor& w, int64_t groups, double eps,
+                              const c10::optional<at::Tensor>& mix, const c10::optional<at::Tensor>& ls1,
+                              const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& pair_slot,
+                              int64_t top, const c10::optional<at::Tensor>& ls2,
+                              const c10::optional<at::Tensor>& extra) {
+  CHECK_DEV(out); CHECK_CONTIG(out); CHECK_F32(residual); CHECK_F32(w);
+  const bool f32 = is_f32(out, "scaled_add_group_rmsnorm");
+  TORCH_CHECK(residual.dim() == 2 && out.sizes() == residual.sizes());
+  const long T = residual.size(0), H = residual.size(1);
+  TORCH_CHECK(groups >= 1 && H % groups == 0 && w.numel() == H && H + groups <= 15000, "group norm shape");
+  if (mix.has_value()) {
+    TORCH_CHECK(mix->scalar_type() == out.scalar_type() && mix->is_contiguous() && mix->sizes() == residual.sizes());
+    TORCH_CHECK(ls1.has_value() && ls1->scalar_type() == at::kFloat && ls1->numel() == H);
+  }
+  if (y.has_value()) {
+    TORCH_CHECK(y->scalar_type() == out.scalar_type() && y->is_contiguous() && y->dim() == 2 && y->size(1) == H);
+    TORCH_CHECK(top >= 1 && pair_slot.has_value() && pair_slot->scalar_type() == at::kInt &&
+                pair_slot->is_contiguous() && pair_slot->numel() >= T * top);
+    TORCH_CHECK(ls2.has_value() && ls2->scalar_type() == at::kFloat && ls2->numel() == H);
+  }
+  if (extra.has_value())
+    TORCH_CHECK(extra->scalar_type() == out.scalar_type() && extra->is_contiguous() && extra->sizes() == residual.sizes());
+  c10::hip::HIPGuardMasqueradingAsCUDA g(out.device());
+  hipserve::launch_scaled_add_group_rmsnorm(
+      out.data_ptr(), residual.data_ptr<float>(), w.data_ptr<float>(), T, H, groups, (float)eps, opt_ptr(mix),
+      (const float*)opt_ptr(ls1), opt_ptr(y), (const int*)opt_ptr(pair_slot), y.has_value() ? top : 0,
+      (const float*)opt_ptr(ls2), opt_ptr(extra), f32, cur_stream());
+}
+
+void latent_prepare(at::Tensor& cq, at::Tensor& cache, const at::Tensor& proj, const at::Tensor& positions,
+                    const at::Tensor& slots, const at::Tensor& q_norm, const at::Tensor& kv_norm,
+                    const at::Tensor& inv_freq, int64_t q_rank, int64_t kv_rank, int64_t rot_dim, double eps) {
+  CHECK_DEV(proj); CHECK_CONTIG(cq); CHECK_CONTIG(cache); CHECK_F32(q_norm); CHECK_F32(kv_norm); CHECK_F32(inv_freq);
+  const bool f32 = is_f32(proj, "latent_prepare");
+  TORCH_CHECK(cq.scalar_type() == proj.scalar_type() && cache.scalar_type() == proj.scalar_type());
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(1) >= q_rank + kv_rank + rot_dim);
+  const long T = proj.size(0);
+  TORCH_CHECK(cq.numel() == T * q_rank && cache.dim() == 3 && cache.size(2) == kv_rank + rot_dim);
+  TORCH_CHECK(positions.scalar_type() == at::kLong && slots.scalar_type() == at::kLong && positions.numel() >= T &&
+              slots.numel() >= T && positions.is_contiguous() && slots.is_contiguous());
+  TORCH_CHECK(q_norm.numel() == q_rank && kv_norm.numel() == kv_rank && 2 * inv_freq.numel() <= rot_dim);
+  c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+  hipserve::launch_latent_prepare(cq.data_ptr(), cache.data_ptr(), proj.data_ptr(), proj.stride(0),
+                                  positions.data_ptr<long>(), slots.data_ptr<long>(), q_norm.data_ptr<float>(),
+                                  kv_norm.data_ptr<float>(), inv_freq.data_ptr<float>(), inv_freq.numel(), T, q_rank,
+                                  kv_rank, rot_dim, (float)eps, f32, cur_stream());
+}
+
+void latent_attention(at::Tensor& o_lat, const at::Tensor& q_abs, const at::Tensor& q, const at::Tensor& proj,
+                      const at::Tensor& cache, const at::Tensor& seq_cu, const at::Tensor& seq_ctx,
+                      const at::Tensor& seq_bt, int64_t seq0, int64_t seq1, int64_t rows_bound, int64_t tq,
+                      const at::Tensor& inv_freq, int64_t heads, int64_t dim, int64_t rot_dim, int64_t kv_rank,
+                      int64_t gate_off, double scale, int64_t window) {
+  CHECK_DEV(q); CHECK_CONTIG(o_lat); CHECK_F32(q_abs); CHECK_CONTIG(q); CHECK_CONTIG(cache); CHECK_F32(inv_freq);
+  CHECK_I32(seq_cu); CHECK_I32(seq_ctx); CHECK_I32(seq_bt);
+  const bool f32 = is_f32(q, "latent_attention");
+  TORCH_CHECK(o_lat.scalar_type() == q.scalar_type() && cache.scalar_type() == q.scalar_type() &&
+              proj.scalar_type() == q.scalar_type());
+  const long T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) == heads * (dim + rot_dim));
+  TORCH_CHECK(q_abs.numel() == heads * T * kv_rank && o_lat.numel() == heads * T * kv_rank);
+  TORCH_CHECK(cache.dim() == 3 && cache.size(2) == kv_rank + rot_dim && kv_rank <= 1024);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T && proj.size(1) >= gate_off + heads);
+  const long nseq = seq_ctx.numel();
+  TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_bt.dim() == 2 && seq_bt.size(0) >= nseq);
+  TORCH_CHECK(0 <= seq0 && seq0 <= seq1 && seq1 <= nseq && rows_bound <= T);
+  TORCH_CHECK(tq == 1 || tq == 2 || tq == 4 || tq == 8 || tq == 16, "tokens per workgroup: 1, 2, 4, 8 or 16");
+  TORCH_CHECK(2 * inv_freq.numel() <= rot_dim);
+  c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
+  hipserve::launch_latent_attention(o_lat.data_ptr(), q_abs.data_ptr<float>(), q.data_ptr(), proj.data_ptr(),
+                                    proj.stride(0), cache.data_ptr(), cache.size(1), seq_cu.data_ptr<int>(),
+                                    seq_ctx.data_ptr<int>(), seq_bt.data_ptr<int>(), seq_bt.size(1), seq0, seq1,
+                                    rows_bound, tq, inv_freq.data_ptr<float>(), inv_freq.numel(), T, heads, dim,
+                                    rot_dim, kv_rank, gate_off, (float)scale, window, f32, cur_stream());
+}
+
+void mingru_scan(at::Tensor& y, at::Tensor& state, const at::Tensor& proj, const at::Tensor& b_z,
+                 const at::Tensor& b_x, const at::Tensor& seq_cu, const at::Tensor& seq_ctx,
+                 const at::Tensor& seq_state, int64_t max_q) {
+  CHECK_DEV(proj); CHECK_CONTIG(proj); CHECK_CONTIG(y); CHECK_F32(state); CHECK_F32(b_z); CHECK_F32(b_x);
+  CHECK_I32(seq_cu); CHECK_I32(seq_ctx); CHECK_I32(seq_state);
+  const bool f32 = is_f32(proj, "mingru_scan");
+  TORCH_CHECK(y.scalar_type() == proj.scalar_type());
+  const long width = state.size(1), nseq = seq_ctx.numel();
+  TORCH_CHECK(proj.dim() == 2 && proj.size(1) == 3 * width && y.numel() == proj.size(0) * width);
+  TORCH_CHECK(b_z.numel() == width && b_x.numel() == width);
+  TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_state.numel() >= nseq);
+  c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+  hipserve::launch_mingru_scan(y.data_ptr(), state.data_ptr<float>(), proj.data_ptr(), b_z.data_ptr<float>(),
+                               b_x.data_ptr<float>(), seq_cu.data_ptr<int>(), seq_ctx.data_ptr<int>(),
+                               seq_state.data_ptr<int>(), nseq, width, max_q, f32, cur_stream());
+}
+
+void moe_align(const at::Tensor& ids, int64_t E, int64_t tile, at::Tensor& slots, at::Tensor& tile_expert,
+               at::Tensor& pair_slot) {
+  CHECK_DEV(ids); CHECK_I32(ids); CHECK_I32(slots); CHECK_I32(tile_expert); CHECK_I32(pair_slot);
+  TORCH_CHECK(E >= 1 && E <= 128, "moe_align: at most 128 experts");
+  TORCH_CHECK(tile == 16 || tile == 32 || tile == 64 || tile == 128 || tile == 256);
+  const int npairs = ids.numel();
+  TORCH_CHECK(slots.numel() >= npairs + E * (tile - 1) && slots.numel() % tile == 0,
+              "slots capacity must cover padding and be a multiple of the tile");
+  TORCH_CHECK(tile_expert.numel() * tile >= slots.numel() && pair_slot.numel() >= npairs);
+  c10::hip::HIPGuardMasqueradingAsCUDA g(ids.device());
+  const int nb = hipserve::moe_align_blocks(npairs);
+  at::Tensor scratch = at::empty({(long)(nb > 1 ? nb : 0) * 128 + 1}, ids.options());  // [hist | tile count]
+  hipserve::launch_moe_align(ids.data_ptr<int>(), npairs, E, tile, slots.data_ptr<int>(), slots.numel(),
+                             tile_expert.data_ptr<int>(), tile_expert.numel(),
+                             scratch.data_ptr<int>() + (scratch.numel() - 1), pair_slot.data_ptr<int>(), nullptr,
+                             cur_stream(), nb > 1 ? scratch.data_ptr<int>() : nullptr);
+}
+
+void expert_gemm(at::Tensor& out, const at::Tensor& x, const at::Tensor& w, const at::Tensor& slots,
+                 const at::Tensor& tile_expert, int64_t tile, int64_t gather_k, bool relu2) {
+  CHECK_DEV(x); CHECK_CONTIG(out); CHECK_CONTIG(w); CHECK_I32(slots); CHECK_I32(tile_expert);
+  const bool f32 = is_f32(x, "expert_gemm");
+  TORCH_CHECK(out.scalar_type() == x.scalar_type() && w.scalar_type() == x.scalar_type());
+  TORCH_CHECK(w.dim() == 3 && x.dim() == 2 && x.stride(1) == 1 && out.dim() == 2);
+  const long N = w.size(1), K = w.size(2), cap = slots.numel();
+  TORCH_CHECK(x.size(1) == K && out.size(1) == N && out.size(0) >= cap);
+  TORCH_CHECK(tile % 32 == 0 && cap % tile == 0 && tile_expert.numel() * tile >= cap, "tiles of a multiple of 32 slots");
+  TORCH_CHECK(gather_k > 0 || x.size(0) >= cap, "ungathered x needs one row per slot");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  hipserve::launch_expert_gemm(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(), slots.data_ptr<int>(),
+                               tile_expert.data_ptr<int>(), cap / tile, tile, gather_k, N, K, relu2, f32, cur_stream());
+}
+
+}  // namespace
+
+TORCH_LIBRARY(hipserve_seq, m) {
+  m.def("scaled_add_group_rmsnorm(Tensor(a!) out, Tensor(b!) residual, Tensor w, int groups, float eps, Tensor? mix, "
+        "Tensor? ls1, Tensor? y, Tensor? pair_slot, int top, Tensor? ls2, Tensor? extra) -> ()");
+  m.def("latent_prepare(Tensor(a!) cq, Tensor(b!) cache, Tensor proj, Tensor positions, Tensor slots, Tensor q_norm, "
+        "Tensor kv_norm, Tensor inv_freq, int q_rank, int kv_rank, int rot_dim, float eps) -> ()");
+  m.def("latent_attention(Tensor(a!) o_lat, Tensor q_abs, Tensor q, Tensor proj, Tensor cache, Tensor seq_cu, "
+        "Tensor seq_ctx, Tensor seq_bt, int seq0, int seq1, int rows_bound, int tq, Tensor inv_freq, int heads, "
+        "int dim, int rot_dim, int kv_rank, int gate_off, float scale, int window) -> ()");
+  m.def("mingru_scan(Tensor(a!) y, Tensor(b!) state, Tensor proj, Tensor b_z, Tensor b_x, Tensor seq_cu, "
+        "Tensor seq_ctx, Tensor seq_state, int max_q) -> ()");
+  m.def("moe_align(Tensor ids, int E, int tile, Tensor(a!) slots, Tensor(b!) tile_expert, Tensor(c!) pair_slot) -> ()");
+  m.def("expert_gemm(Tensor(a!) out, Tensor x, Tensor w, Tensor slots, Tensor tile_expert, int tile, int gather_k, "
+        "bool relu2) -> ()");
+}
+
+TORCH_LIBRARY_IMPL(hipserve_seq, CUDA, m) {
+  m.impl("scaled_add_group_rmsnorm", &scaled_add_group_rmsnorm);
+  m.impl("latent_prepare", &latent_prepare);
+  m.impl("latent_attention", &latent_attention);
+  m.impl("mingru_scan", &mingru_scan);
+  m.impl("moe_align", &moe_align);
+  m.impl("expert_gemm", &expert_gemm);
+}

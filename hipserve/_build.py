@@ -33,7 +33,17 @@ HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
     "-munsafe-fp-atomics", "-ffp-contract=fast", "-Wno-unused-result",
     "-Wno-unused-variable",
+    # no packed-fp32 instructions from ordinary float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+# kernel libraries: name -> (shared object, kernel sources, host bindings). "core" is every
+# dense-transformer / sampling / quantisation kernel; "seq" the layer-list decoders' kernels
+# (plus the expert alignment of moe.hip), so a model of those designs builds only what it runs.
+LIBS = {
+    "core": ("_C.so", ["kernels/*.hip"], "torch_bindings.cpp"),
+    "seq": ("_C_seq.so", ["kernels/seq/*.hip", "kernels/moe.hip"], "seq_bindings.cpp"),
+}
 
 
 def _torch_paths():
@@ -83,17 +93,20 @@ def _compile(src, obj, cmd, want):
     return src, out
 
 
-def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> str:
-    """Build hipserve/_C.so (gfx950 kernels + torch op registrations)."""
+def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False, lib: str = "core") -> str:
+    """Build one kernel library of ``LIBS`` (gfx950 kernels + torch op registrations):
+    ``core`` = hipserve/_C.so, ``seq`` = hipserve/_C_seq.so."""
     if not os.path.exists(HIPCC):
         raise RuntimeError(f"hipcc not found at {HIPCC}")
+    so_name, patterns, bindings = LIBS[lib]
     os.makedirs(BUILD, exist_ok=True)
     inc, libdir, abi = _torch_paths()
-    hdrs = _headers()
+    hdrs = _headers() + sorted(glob.glob(os.path.join(CSRC, "kernels", "**", "*.h"), recursive=True))
     inc_flags = ["-I", os.path.join(CSRC, "include")]
     tasks = []
     objs = []
-    for src in sorted(glob.glob(os.path.join(CSRC, "kernels", "*.hip"))):
+    srcs = sorted(p for pat in patterns for p in glob.glob(os.path.join(CSRC, pat)))
+    for src in srcs:
         obj = os.path.join(BUILD, os.path.basename(src) + ".o")
         flags = HIP_FLAGS + inc_flags
         want = _stamp([src] + hdrs, flags)
@@ -101,8 +114,8 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
         if force or _needs(obj, [src] + hdrs, flags):
             tasks.append((src, obj, [HIPCC, *flags, "-c", src, "-o", obj], want))
     # host-only translation unit with the torch registrations
-    bsrc = os.path.join(CSRC, "torch_bindings.cpp")
-    bobj = os.path.join(BUILD, "torch_bindings.o")
+    bsrc = os.path.join(CSRC, bindings)
+    bobj = os.path.join(BUILD, os.path.splitext(bindings)[0] + ".o")
     bflags = ["-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
               f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-I", os.path.join(ROCM, "include"),
               *inc_flags] + [x for p in inc for x in ("-isystem", p)]
@@ -119,7 +132,7 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
                     print(f"[hipserve build] {os.path.relpath(src, ROOT)}", flush=True)
                     if out.strip():
                         print(out, flush=True)
-    so = os.path.join(PKG, "_C.so")
+    so = os.path.join(PKG, so_name)
     if tasks or not os.path.exists(so):
         # Link with the host toolchain and WITHOUT -lamdhip64: the HIP runtime
         # symbols resolve through libtorch_hip's own libamdhip64, so the process
@@ -135,7 +148,7 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False) -> 
         missing = [ln.split(None, 1)[-1] for ln in und.stdout.splitlines() if "hipserve::" in ln]
         if missing:
             os.remove(so + ".tmp")
-            raise RuntimeError("hipserve/_C.so has undefined hipserve symbols: " + "; ".join(missing))
+            raise RuntimeError(f"hipserve/{so_name} has undefined hipserve symbols: " + "; ".join(missing))
         os.replace(so + ".tmp", so)
     return so
 
@@ -204,6 +217,7 @@ def build_all(force: bool = False, jobs: int | None = None, verbose: bool = True
     jobs = jobs or int(os.environ.get("MAX_JOBS", "8"))
     rt = build_runtime(force=force, verbose=verbose)
     so = build_kernels(force=force, jobs=jobs, verbose=verbose)
+    build_kernels(force=force, jobs=jobs, verbose=verbose, lib="seq")
     return so, rt
 
 

@@ -1,7 +1,8 @@
 """hipserve op library.
 
 ``KernelOps`` calls the hand-written gfx950 kernels in ``hipserve/_C.so``
-(``torch.ops.hipserve.*``). ``ReferenceOps`` is the plain-PyTorch oracle used by
+(``torch.ops.hipserve.*``) and, for the layer-list decoders, ``hipserve/_C_seq.so``
+(``torch.ops.hipserve_seq.*``); each library is loaded at the first use of one of its kernels. ``ReferenceOps`` is the plain-PyTorch oracle used by
 the CPU plumbing engine and by the numerics tests. The choice is made ONCE, when
 an engine is built for a device — never per call. On a GPU device the native
 library is mandatory: a missing/unloadable ``_C.so`` raises instead of silently
@@ -16,9 +17,12 @@ import torch
 
 from . import reference as ref
 
-_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "_C.so")
+_PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_LIB = os.path.join(_PKG, "_C.so")
+_LIB_SEQ = os.path.join(_PKG, "_C_seq.so")  # the layer-list decoders' kernels (torch.ops.hipserve_seq)
 _lock = threading.Lock()
 _loaded = False
+_loaded_seq = False
 
 
 def library_path() -> str:
@@ -43,6 +47,22 @@ def load_library(build_if_missing: bool = False) -> str:
         return _LIB
 
 
+def load_seq_library() -> str:
+    """Load hipserve/_C_seq.so into torch.ops (idempotent); built first when it is missing
+    (a few hipcc seconds: four kernel files)."""
+    global _loaded_seq
+    with _lock:
+        if _loaded_seq:
+            return _LIB_SEQ
+        if not os.path.exists(_LIB_SEQ):
+            from .._build import build_kernels
+
+            build_kernels(lib="seq")
+        torch.ops.load_library(_LIB_SEQ)
+        _loaded_seq = True
+        return _LIB_SEQ
+
+
 def native_available() -> bool:
     try:
         load_library()
@@ -57,8 +77,23 @@ class KernelOps:
     name = "hip"
 
     def __init__(self):
-        load_library()
-        self._op = torch.ops.hipserve
+        self._core = None
+        self._seq_ops = None
+
+    @property
+    def _op(self):
+        """torch.ops.hipserve, loaded at the first use of a core kernel (a missing _C.so raises there)."""
+        if self._core is None:
+            load_library(build_if_missing=os.environ.get("HIPSERVE_BUILD_ON_DEMAND") == "1")
+            self._core = torch.ops.hipserve
+        return self._core
+
+    @property
+    def _seq(self):
+        if self._seq_ops is None:
+            load_seq_library()
+            self._seq_ops = torch.ops.hipserve_seq
+        return self._seq_ops
 
     def rmsnorm(self, out, x, w, eps, out8=None):
         """out8: (e4m3 [rows, hidden] uint8, scales fp32 [rows]) per-token FP8 copy of out."""
@@ -141,6 +176,42 @@ class KernelOps:
         cu, tiles = meta
         self._op.vision_attention(out, qkv, cos_sin, cu, tiles, nh, D, scale)
         return out
+
+
+    # ---- layer-list decoders (csrc/kernels/seq/*.hip; bf16 or true fp32 activations)
+    def scaled_add_group_rmsnorm(self, out, residual, w, groups, eps, mix=None, ls1=None, y=None, pair_slot=None,
+                                 top=0, ls2=None, extra=None):
+        self._seq.scaled_add_group_rmsnorm(out, residual, w, groups, eps, mix, ls1, y, pair_slot, top, ls2, extra)
+        return out
+
+    def latent_prepare(self, cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
+                       rot_dim, eps):
+        self._seq.latent_prepare(cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
+                                 rot_dim, eps)
+
+    LATENT_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x up to 4 heads = 16 waves)
+
+    def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
+                         gate_off, scale, window):
+        """Prompt portions (the step's first sequences) run several tokens per workgroup, decode
+        rows one token x up to 16 heads; both on the same kernel."""
+        nseq = meta.seq_ctx.shape[0]
+        npf = nseq - meta.num_decode
+        for s0, s1, rows, tq in ((0, npf, meta.num_prefill_tokens, self.LATENT_PREFILL_TQ),
+                                 (npf, nseq, meta.num_decode, 1)):
+            if s1 > s0:
+                self._seq.latent_attention(o_lat, q_abs, q, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt,
+                                           s0, s1, rows, tq, inv_freq, heads, dim, rot_dim, kv_rank, gate_off,
+                                           scale, window)
+
+    def mingru_scan(self, y, state, proj, b_z, b_x, meta):
+        self._seq.mingru_scan(y, state, proj, b_z, b_x, meta.seq_cu, meta.seq_ctx, meta.seq_state, meta.max_q)
+
+    def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
+        self._seq.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
+
+    def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
+        self._seq.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
 
 
 class ReferenceOps:
