@@ -77,6 +77,13 @@ def parse():
     ap.add_argument("--tp-steps", type=int, default=2)
     ap.add_argument("--tp-warmup", type=int, default=1)
     ap.add_argument("--tp-budget-s", type=float, default=150.0)
+    ap.add_argument("--layer-compare", action="store_true",
+                    help="instead of the headline benchmark: prefill / decode tok/s of the Kesirax decoder "
+                         "beside a Mixtral-style model of equal size (hipserve/bench/layer_compare.py)")
+    ap.add_argument("--layer-sizes", default="", help="with --layer-compare: sizes, comma separated (default: all)")
+    ap.add_argument("--layer-batch", type=int, default=16)
+    ap.add_argument("--layer-prompt", type=int, default=2048)
+    ap.add_argument("--layer-new", type=int, default=64)
     ap.add_argument("--result-file", default=None, help=argparse.SUPPRESS)  # child -> parent
     ap.add_argument("--deadline", type=float, default=None, help=argparse.SUPPRESS)
     ap.add_argument("--request-rate", type=float, default=None,
@@ -278,6 +285,10 @@ def orchestrate(args) -> int:
 
 def main():
     args = parse()
+    if args.layer_compare:  # its own single-GPU workload; the headline contract below is untouched
+        from hipserve.bench.layer_compare import main as layer_compare
+
+        sys.exit(layer_compare(args))
     world_env = os.environ.get("WORLD_SIZE")
     if world_env is None and args.gpus > 1:
         sys.exit(_self_launch(args))

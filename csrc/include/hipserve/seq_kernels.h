@@ -30,6 +30,19 @@ void launch_latent_attention(void* o_lat, const float* q_abs, const void* q, con
                              const float* inv_freq, int nfreq, int T, int heads, int dim, int rot_dim, int kv_rank,
                              int gate_off, float scale, int window, bool f32, hipStream_t s);
 
+// bf16 prompt portions on the matrix cores (latent_attention_mfma.hip): qc[heads, T, kv_rank + rot_dim] =
+// [q_abs | RoPE(q rotary part)] as bf16, then the attention on 64-row x 32-key MFMA tiles. nparts > 1
+// (rows of one token each, rows_bound of them from batch row row_base on): the keys are split into runs of
+// part_keys (a multiple of 32) over ws_acc [nparts, heads, rows_bound, kv_rank] / ws_ml [.., 2] and merged.
+void launch_latent_q_cat(void* qc, const float* q_abs, const void* q, const long* positions, const float* inv_freq,
+                         int nfreq, int T, int heads, int dim, int rot_dim, int kv_rank, hipStream_t s);
+bool latent_attention_mfma_ok(int kv_rank, int rot_dim);
+void launch_latent_attention_mfma(void* o_lat, const void* qc, const void* proj, long proj_ld, const void* cache,
+                                  int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
+                                  int bt_width, int seq0, int seq1, int rows_bound, int T, int heads, int rot_dim,
+                                  int kv_rank, int gate_off, float scale, int window, int nparts, int part_keys,
+                                  float* ws_acc, float* ws_ml, int row_base, hipStream_t s);
+
 // minGRU over the step's rows of every sequence, from / to its fp32 state slot.
 void launch_mingru_scan(void* y, float* state, const void* proj, const float* b_z, const float* b_x,
                         const int* seq_cu, const int* seq_ctx, const int* seq_state, int nseq, int width, int max_q,

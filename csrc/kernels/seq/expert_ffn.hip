@@ -68,11 +68,89 @@ __global__ __launch_bounds__(256) void expert_gemm_kernel(T* __restrict__ out, c
   }
 }
 
+// bf16 on the matrix cores: a workgroup (4 waves) computes [16 ST slots x 128 columns]; wave w owns
+// columns 32 w .. 32 w + 31. Operands go from global memory straight into the MFMA registers (16 bytes
+// per lane and step: 8 consecutive k of one W row / one x row); W rows are read once per slot tile, the
+// x rows of the tile are shared by the four waves through L1. Needs K % 8 == 0, N % 8 == 0.
+template <int ST>
+__global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(
+    unsigned short* __restrict__ out, const unsigned short* __restrict__ x, long x_ld,
+    const unsigned short* __restrict__ w, const int* __restrict__ slots, const int* __restrict__ tile_expert,
+    int gather_k, int N, int K, int relu2) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int slot0 = blockIdx.y * 16 * ST;
+  const int n0 = blockIdx.x * 128 + 32 * wave;
+  if (n0 >= N) return;
+  const unsigned short* xr[ST];
+  bool live[ST];
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    const int slot = slot0 + 16 * st + c;
+    const int p = slots[slot];
+    live[st] = p >= 0;
+    xr[st] = x + (p < 0 ? 0 : (gather_k > 0 ? (long)(p / gather_k) : (long)slot)) * x_ld + 8 * g;
+  }
+  const unsigned short* wr[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) wr[nt] = w + ((long)e * N + min(n0 + 16 * nt + c, N - 1)) * K + 8 * g;
+  f32x4 acc[2][ST];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int st = 0; st < ST; ++st) acc[nt][st] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const u16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 2
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool in = k0 + 8 * g < K;
+    u16x8 a[2], b[ST];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) a[nt] = in ? *reinterpret_cast<const u16x8*>(wr[nt] + k0) : zero;
+#pragma unroll
+    for (int st = 0; st < ST; ++st) b[st] = (in && live[st]) ? *reinterpret_cast<const u16x8*>(xr[st] + k0) : zero;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int st = 0; st < ST; ++st)
+        acc[nt][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[nt]),
+                                                              __builtin_bit_cast(bf16x8, b[st]), acc[nt][st], 0, 0, 0);
+  }
+  // lane (c, g): columns n0 + 16 nt + 4 g .. + 3 of slot 16 st + c
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    if (!live[st]) continue;
+    const long slot = slot0 + 16 * st + c;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int n = n0 + 16 * nt + 4 * g;
+      if (n >= N) continue;  // N % 8 == 0: the four columns are inside together
+      u16x4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v = acc[nt][st][j];
+        if (relu2) { v = fmaxf(v, 0.f); v *= v; }
+        o[j] = f32_to_bf16(v);
+      }
+      *reinterpret_cast<u16x4*>(out + slot * N + n) = o;
+    }
+  }
+}
+
 }  // namespace
 
 void launch_expert_gemm(void* out, const void* x, long x_ld, const void* w, const int* slots, const int* tile_expert,
                         int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, bool f32, hipStream_t s) {
   if (ntiles_cap <= 0) return;
+  if (!f32 && K % 8 == 0 && N % 8 == 0 && x_ld % 8 == 0 && (tile == 32 || tile == 64)) {
+    dim3 mg((N + 127) / 128, ntiles_cap);
+    auto o = (unsigned short*)out;
+    auto xi = (const unsigned short*)x, wi = (const unsigned short*)w;
+    if (tile == 32) expert_gemm_mfma_kernel<2><<<mg, 256, 0, s>>>(o, xi, x_ld, wi, slots, tile_expert, gather_k, N, K, relu2);
+    else expert_gemm_mfma_kernel<4><<<mg, 256, 0, s>>>(o, xi, x_ld, wi, slots, tile_expert, gather_k, N, K, relu2);
+    return;
+  }
   dim3 grid((N + kTN - 1) / kTN, (long)ntiles_cap * tile / kTM);
   if (f32)
     expert_gemm_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)x, x_ld, (const float*)w, slots,

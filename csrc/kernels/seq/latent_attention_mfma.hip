@@ -1,0 +1,350 @@
+// Latent attention for prompt portions on the matrix cores (bf16 activations and cache).
+//
+// latent_q_cat: the query rows the attention multiplies with the cached rows,
+//   qc[h, t, :] = [ q_abs[h, t, :kv_rank] | RoPE(q[t, h, dim:]) ]  (bf16, Dk = kv_rank + rot_dim).
+//
+// latent_attention_mfma: a workgroup (4 waves) owns 64 (token, head) rows of one sequence, tokens
+// consecutive, so all rows share one run of keys. Per 32-key tile:
+//   1. the tile's cache rows [32][Dk] go to LDS row-major; wave w computes S = K . Q^T for its 16 rows
+//      (mfma_f32_16x16x32_bf16, the Q operands stay in registers) and writes it to LDS as fp32;
+//   2. four threads per row do the masked online softmax in fp32 (max, exp, sum, rescale factor) and
+//      write P as bf16;
+//   3. every wave owns a slice of the latent dims for ALL 64 rows: acc = acc * alpha + V^T . P^T. The
+//      contraction index is the key, so the V operand is read column-wise from the same row-major K
+//      tile (eight 2-byte LDS reads per operand; the MFMA's k slots are dealt to keys 4 e + g so that
+//      the four rows read together hit disjoint banks, and P is stored in that key order).
+// Decode rows (one token, many keys) split their keys over grid.z; latent_attention_reduce merges the
+// runs' (max, sum, output).
+// The output (latent space, times the head's sigmoid gate, over the softmax sum) is written as bf16.
+#include "seq_common.h"
+#include "hipserve/seq_kernels.h"
+
+namespace hipserve {
+namespace {
+
+__global__ __launch_bounds__(256) void latent_q_cat_kernel(unsigned short* __restrict__ qc,
+                                                           const float* __restrict__ q_abs,
+                                                           const unsigned short* __restrict__ q,
+                                                           const long* __restrict__ positions,
+                                                           const float* __restrict__ inv_freq, int nfreq, int T,
+                                                           int heads, int dim, int rot_dim, int kv_rank) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int Dk = kv_rank + rot_dim;
+  unsigned short* dst = qc + ((long)h * T + t) * Dk;
+  const float* qa = q_abs + ((long)h * T + t) * kv_rank;
+  for (int e = threadIdx.x; e < kv_rank; e += 256) dst[e] = f32_to_bf16(qa[e]);
+  const unsigned short* qr = q + (long)t * heads * (dim + rot_dim) + (long)h * (dim + rot_dim) + dim;
+  const float pos = (float)positions[t];
+  for (int e = threadIdx.x; e < rot_dim; e += 256) {
+    float v;
+    if (e < 2 * nfreq) {
+      const int i = e < nfreq ? e : e - nfreq;
+      float sn, cs;
+      sincosf(pos * inv_freq[i], &sn, &cs);
+      const float u = bf16_to_f32(qr[i]), w = bf16_to_f32(qr[i + nfreq]);
+      v = e < nfreq ? u * cs - w * sn : w * cs + u * sn;
+    } else {
+      v = bf16_to_f32(qr[e]);
+    }
+    dst[kv_rank + e] = f32_to_bf16(v);
+  }
+}
+
+constexpr int kRows = 64;   // (token, head) rows per workgroup
+constexpr int kKeys = 32;   // keys per tile
+constexpr int kPLd = 40;    // P tile row stride (elements): 16-byte aligned rows, padded
+
+HS_DEVICE bool find_tile64(const int* __restrict__ seq_cu, int seq0, int seq1, int tq, int wg, int& s, int& tok0) {
+  int acc = 0;
+  for (int i = seq0; i < seq1; ++i) {
+    const int n = seq_cu[i + 1] - seq_cu[i];
+    const int nt = (n + tq - 1) / tq;
+    if (wg < acc + nt) {
+      s = i;
+      tok0 = (wg - acc) * tq;
+      return true;
+    }
+    acc += nt;
+  }
+  return false;
+}
+
+// K tile row stride: 32 KS + pad with stride / 2 = 8 (mod 32) dwords, so that the four key rows a wave
+// reads together in the P . V operand loads fall into disjoint LDS banks; a multiple of 8 elements.
+template <int KS> struct KtLd { static constexpr int v = KS * 32 + ((KS & 1) ? 48 : 16); };
+
+// KS: 32-dim steps of a cache row (Dk <= 32 KS); NPW: 16-dim output tiles per wave (kv_rank <= 64 NPW).
+// grid.z > 1 splits the keys of a row into runs of part_keys; the runs' unnormalised outputs and
+// (max, sum) go to ws_acc / ws_ml for latent_attention_reduce (decode rows: many keys, few rows).
+template <int KS, int NPW>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    unsigned short* __restrict__ o_lat, const unsigned short* __restrict__ qc, const unsigned short* __restrict__ proj,
+    long proj_ld, const unsigned short* __restrict__ cache, int block_size, const int* __restrict__ seq_cu,
+    const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
+    int T_rows, int heads, int rot_dim, int kv_rank, int gate_off, float scale, int window, int part_keys,
+    float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows) {
+  constexpr int kLd = KtLd<KS>::v;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned short* kt = reinterpret_cast<unsigned short*>(smem);                    // [32][kLd] bf16 cache rows
+  float* s_lds = reinterpret_cast<float*>(smem + kKeys * kLd * 2);                 // [64][32] fp32 scores
+  unsigned short* p_lds = reinterpret_cast<unsigned short*>(s_lds + kRows * kKeys);  // [64][kPLd] bf16, keys permuted
+  float* alpha = reinterpret_cast<float*>(p_lds + kRows * kPLd);                   // [64]
+  float* m_run = alpha + kRows;                                                    // [64]
+  float* l_run = m_run + kRows;                                                    // [64]
+  int s, tok0;
+  if (!find_tile64(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) return;
+  const int Dk = kv_rank + rot_dim;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0, ctx = seq_ctx[s];
+  const int ntok = min(tq, n - tok0);
+  const int h0 = blockIdx.y * hc, nh = min(hc, heads - h0);
+  const int p_first = ctx - n + tok0, p_last = p_first + ntok - 1;
+  const int lo_all = window > 0 ? max(0, p_first - window + 1) : 0;
+  const int lo = lo_all + blockIdx.z * part_keys;
+  const int hi = gridDim.z > 1 ? min(p_last, lo + part_keys - 1) : p_last;
+  // Q operands of this wave's 16 rows (row = 16 wave + c): dims 32 ks + 8 g .. + 7
+  bf16x8 qf[KS];
+  {
+    const int r = 16 * wave + c;
+    const int rt = r / hc, rh = r % hc;
+    const bool act = rt < ntok && rh < nh;
+    const unsigned short* src = qc + ((long)(h0 + (act ? rh : 0)) * T_rows + r0 + tok0 + (act ? rt : 0)) * Dk;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = 32 * ks + 8 * g;
+      u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (act && d < Dk) v = *reinterpret_cast<const u16x8*>(src + d);
+      qf[ks] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  if (tid < kRows) { m_run[tid] = -INFINITY; l_run[tid] = 0.f; }
+  f32x4 acc[4][NPW];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int j = 0; j < NPW; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int ntiles_dv = (kv_rank + 15) / 16;
+  const int chunks = Dk / 8;  // 16-byte chunks of a cache row
+  // tile fill: 8 threads per key, each its key's chunks fk, fk + 8, ...
+  const int fkey = tid >> 3, fk = tid & 7;
+  // softmax: 4 threads per row; thread `part` owns the keys 4 e + part (e = 0..7) of the tile
+  const int sr = tid >> 2, part = tid & 3;
+  const int srt = sr / hc, srh = sr % hc;
+  const bool sact = srt < ntok && srh < nh;
+  const int spos = p_first + srt;
+  const int s_lo = window > 0 ? max(0, spos - window + 1) : 0;
+  for (int j0 = lo; j0 <= hi; j0 += kKeys) {
+    __syncthreads();  // the previous tile's reads of the K tile (P . V) are done
+    {
+      const int j = j0 + fkey;
+      const bool in = j <= hi;
+      const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dk : 0;
+      for (int ch = fk; ch < KS * 4; ch += 8) {  // zero past Dk and past the last key
+        u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (in && ch < chunks) v = *reinterpret_cast<const u16x8*>(cache + kr + 8 * ch);
+        *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = v;
+      }
+    }
+    __syncthreads();
+    // 1. S^T tiles: a = keys (16 per tile), b = this wave's 16 query rows
+    f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const u16x8 a = *reinterpret_cast<const u16x8*>(kt + (16 * nt + c) * kLd + 32 * ks + 8 * g);
+        sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[ks], sc[nt], 0, 0, 0);
+      }
+    }
+    // lane (c, g) holds keys 16 nt + 4 g .. + 3 of row 16 wave + c
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+      *reinterpret_cast<f32x4*>(s_lds + (16 * wave + c) * kKeys + 16 * nt + 4 * g) = sc[nt];
+    __syncthreads();
+    // 2. online softmax in fp32; P as bf16 with key kk at position 8 (kk % 4) + kk / 4 (the MFMA's k order below)
+    {
+      float v[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int kk = 4 * e + part;
+        const int j = j0 + kk;
+        const bool vis = sact && j <= hi && j <= spos && j >= s_lo;
+        v[e] = vis ? s_lds[sr * kKeys + kk] * scale : -INFINITY;
+        mx = fmaxf(mx, v[e]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      const float mo = m_run[sr];
+      const float mn = fmaxf(mo, mx);
+      float sum = 0.f;
+      u16x8 pk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = (v[e] > -INFINITY) ? expf(v[e] - mn) : 0.f;
+        const unsigned short pb = f32_to_bf16(p);
+        pk[e] = pb;
+        sum += bf16_to_f32(pb);  // the sum of the weights that are actually multiplied
+      }
+      sum += __shfl_xor(sum, 1, 64);
+      sum += __shfl_xor(sum, 2, 64);
+      *reinterpret_cast<u16x8*>(p_lds + sr * kPLd + 8 * part) = pk;
+      if (part == 0) {
+        const float al = (mn > -INFINITY) ? expf(mo - mn) : 1.f;  // mo = -inf: 0
+        alpha[sr] = al;
+        l_run[sr] = l_run[sr] * al + sum;
+        m_run[sr] = mn;
+      }
+    }
+    __syncthreads();
+    // 3. acc[rows][dims] = acc * alpha + V^T . P^T: a = 16 latent dims, b = 16 rows; the MFMA's k slot
+    //    (g, e) is key 4 e + g, read column-wise from the row-major K tile
+    bf16x8 pb[4];
+    float al[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      pb[mt] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(p_lds + (16 * mt + c) * kPLd + 8 * g));
+      al[mt] = alpha[16 * mt + c];
+    }
+#pragma unroll
+    for (int j = 0; j < NPW; ++j) {
+      const int nt = wave + 4 * j;
+      if (nt < ntiles_dv) {
+        u16x8 a;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] = kt[(4 * e + g) * kLd + 16 * nt + c];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+          acc[mt][j] *= al[mt];
+          acc[mt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb[mt], acc[mt][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const bool partial = gridDim.z > 1;
+  if (tid < kRows) {  // alpha <- gate / softmax sum of the row (1 for partial results)
+    const int rt = tid / hc, rh = tid % hc;
+    const bool act = rt < ntok && rh < nh;
+    float f = 0.f;
+    if (act && partial) {
+      f = 1.f;
+      const long wrow = (long)blockIdx.z * heads * ws_rows + (long)(h0 + rh) * ws_rows + (r0 + tok0 + rt - row_base);
+      ws_ml[2 * wrow] = m_run[tid];
+      ws_ml[2 * wrow + 1] = l_run[tid];
+    } else if (act && l_run[tid] > 0.f) {
+      const float gt = bf16_to_f32(proj[(long)(r0 + tok0 + rt) * proj_ld + gate_off + h0 + rh]);
+      f = sigmoid_f(gt) / l_run[tid];
+    }
+    alpha[tid] = f;
+  }
+  __syncthreads();
+  // lane (c, g) holds latent dims 16 nt + 4 g .. + 3 of row 16 mt + c
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int r = 16 * mt + c;
+    const int rt = r / hc, rh = r % hc;
+    if (!(rt < ntok && rh < nh)) continue;
+    const float f = alpha[r];
+    const long trow = r0 + tok0 + rt;
+#pragma unroll
+    for (int j = 0; j < NPW; ++j) {
+      const int d = 16 * (wave + 4 * j) + 4 * g;
+      if (d >= kv_rank) continue;  // kv_rank % 8 == 0: the four dims are inside together
+      if (partial) {
+        float* dst = ws_acc + (((long)blockIdx.z * heads + h0 + rh) * ws_rows + (trow - row_base)) * kv_rank + d;
+        *reinterpret_cast<f32x4*>(dst) = acc[mt][j];
+      } else {
+        u16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(acc[mt][j][e] * f);
+        *reinterpret_cast<u16x4*>(o_lat + ((long)(h0 + rh) * T_rows + trow) * kv_rank + d) = o;
+      }
+    }
+  }
+}
+
+// o_lat[h, row_base + r, :] = sum_p acc_p e^(m_p - M) / sum_p l_p e^(m_p - M) * sigmoid(gate)
+__global__ __launch_bounds__(128) void latent_attention_reduce_kernel(
+    unsigned short* __restrict__ o_lat, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
+    const unsigned short* __restrict__ proj, long proj_ld, int gate_off, int nparts, int heads, int ws_rows,
+    int row_base, int T_rows, int kv_rank) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  float M = -INFINITY;
+  for (int p = 0; p < nparts; ++p) M = fmaxf(M, ws_ml[2 * (((long)p * heads + h) * ws_rows + r)]);
+  float L = 0.f;
+  for (int p = 0; p < nparts; ++p) {
+    const long w = ((long)p * heads + h) * ws_rows + r;
+    const float m = ws_ml[2 * w];
+    if (m > -INFINITY) L += ws_ml[2 * w + 1] * expf(m - M);
+  }
+  const long trow = row_base + r;
+  const float gate = sigmoid_f(bf16_to_f32(proj[trow * proj_ld + gate_off + h]));
+  const float f = L > 0.f ? gate / L : 0.f;
+  for (int d = threadIdx.x; d < kv_rank; d += 128) {
+    float o = 0.f;
+    for (int p = 0; p < nparts; ++p) {
+      const long w = ((long)p * heads + h) * ws_rows + r;
+      const float m = ws_ml[2 * w];
+      if (m > -INFINITY) o += ws_acc[w * kv_rank + d] * expf(m - M);
+    }
+    o_lat[((long)h * T_rows + trow) * kv_rank + d] = f32_to_bf16(o * f);
+  }
+}
+
+template <int KS, int NPW>
+void launch_mfma(unsigned short* o_lat, const unsigned short* qc, const unsigned short* proj, long proj_ld,
+                 const unsigned short* cache, int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
+                 int bt_width, int seq0, int seq1, int rows_bound, int T, int heads, int rot_dim, int kv_rank,
+                 int gate_off, float scale, int window, int nparts, int part_keys, float* ws_acc, float* ws_ml,
+                 int row_base, hipStream_t s) {
+  constexpr int kLd = KtLd<KS>::v;
+  constexpr size_t smem = kKeys * kLd * 2 + kRows * kKeys * 4 + kRows * kPLd * 2 + 3 * kRows * 4;
+  static_assert(smem <= 64 * 1024, "LDS");
+  const int hc = min(heads, kRows);
+  // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the 64 rows
+  const int tq = nparts > 1 ? 1 : kRows / hc;
+  dim3 grid(rows_bound / tq + (seq1 - seq0), (heads + hc - 1) / hc, nparts);
+  latent_attention_mfma_kernel<KS, NPW><<<grid, 256, smem, s>>>(
+      o_lat, qc, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, T, heads,
+      rot_dim, kv_rank, gate_off, scale, window, part_keys, ws_acc, ws_ml, row_base, rows_bound);
+  if (nparts > 1)
+    latent_attention_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(o_lat, ws_acc, ws_ml, proj, proj_ld, gate_off,
+                                                                         nparts, heads, rows_bound, row_base, T,
+                                                                         kv_rank);
+}
+
+}  // namespace
+
+void launch_latent_q_cat(void* qc, const float* q_abs, const void* q, const long* positions, const float* inv_freq,
+                         int nfreq, int T, int heads, int dim, int rot_dim, int kv_rank, hipStream_t s) {
+  if (T <= 0) return;
+  latent_q_cat_kernel<<<dim3(T, heads), 256, 0, s>>>((unsigned short*)qc, q_abs, (const unsigned short*)q, positions,
+                                                     inv_freq, nfreq, T, heads, dim, rot_dim, kv_rank);
+}
+
+bool latent_attention_mfma_ok(int kv_rank, int rot_dim) {
+  const int Dk = kv_rank + rot_dim;
+  return kv_rank % 8 == 0 && rot_dim % 8 == 0 && kv_rank <= 512 && Dk <= 640;
+}
+
+void launch_latent_attention_mfma(void* o_lat, const void* qc, const void* proj, long proj_ld, const void* cache,
+                                  int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
+                                  int bt_width, int seq0, int seq1, int rows_bound, int T, int heads, int rot_dim,
+                                  int kv_rank, int gate_off, float scale, int window, int nparts, int part_keys,
+                                  float* ws_acc, float* ws_ml, int row_base, hipStream_t s) {
+  if (seq1 <= seq0 || rows_bound <= 0) return;
+  const int Dk = kv_rank + rot_dim;
+#define HS_LA(KS, NPW)                                                                                              \
+  launch_mfma<KS, NPW>((unsigned short*)o_lat, (const unsigned short*)qc, (const unsigned short*)proj, proj_ld,     \
+                       (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,      \
+                       rows_bound, T, heads, rot_dim, kv_rank, gate_off, scale, window, nparts, part_keys, ws_acc,   \
+                       ws_ml, row_base, s)
+  if (kv_rank <= 128 && Dk <= 192) HS_LA(6, 2);
+  else if (kv_rank <= 256 && Dk <= 320) HS_LA(10, 4);
+  else HS_LA(20, 8);
+#undef HS_LA
+}
+
+}  // namespace hipserve

@@ -101,6 +101,57 @@ void latent_attention(at::Tensor& o_lat, const at::Tensor& q_abs, const at::Tens
                                     rot_dim, kv_rank, gate_off, (float)scale, window, f32, cur_stream());
 }
 
+// bf16 prompt portions on the matrix cores: qc (scratch) [heads, T, kv_rank + rot_dim] is filled here.
+void latent_attention_mfma(at::Tensor& o_lat, at::Tensor& qc, const at::Tensor& q_abs, const at::Tensor& q,
+                           const at::Tensor& proj, const at::Tensor& positions, const at::Tensor& cache,
+                           const at::Tensor& seq_cu, const at::Tensor& seq_ctx, const at::Tensor& seq_bt, int64_t seq0,
+                           int64_t seq1, int64_t rows_bound, const at::Tensor& inv_freq, int64_t heads, int64_t dim,
+                           int64_t rot_dim, int64_t kv_rank, int64_t gate_off, double scale, int64_t window,
+                           int64_t nparts, int64_t part_keys, const c10::optional<at::Tensor>& ws_acc,
+                           const c10::optional<at::Tensor>& ws_ml, int64_t row_base, bool fill_qc) {
+  CHECK_DEV(q); CHECK_CONTIG(o_lat); CHECK_CONTIG(qc); CHECK_F32(q_abs); CHECK_CONTIG(q); CHECK_CONTIG(cache);
+  CHECK_F32(inv_freq); CHECK_I32(seq_cu); CHECK_I32(seq_ctx); CHECK_I32(seq_bt);
+  TORCH_CHECK(q.scalar_type() == at::kBFloat16 && o_lat.scalar_type() == at::kBFloat16 &&
+              qc.scalar_type() == at::kBFloat16 && cache.scalar_type() == at::kBFloat16 &&
+              proj.scalar_type() == at::kBFloat16, "latent_attention_mfma: bf16 only");
+  TORCH_CHECK(hipserve::latent_attention_mfma_ok(kv_rank, rot_dim), "latent_attention_mfma: unsupported latent sizes");
+  const long T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) == heads * (dim + rot_dim));
+  TORCH_CHECK(q_abs.numel() == heads * T * kv_rank && o_lat.numel() == heads * T * kv_rank &&
+              qc.numel() == heads * T * (kv_rank + rot_dim));
+  TORCH_CHECK(cache.dim() == 3 && cache.size(2) == kv_rank + rot_dim);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T && proj.size(1) >= gate_off + heads);
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.is_contiguous() && positions.numel() >= T);
+  const long nseq = seq_ctx.numel();
+  TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_bt.dim() == 2 && seq_bt.size(0) >= nseq);
+  TORCH_CHECK(0 <= seq0 && seq0 <= seq1 && seq1 <= nseq && rows_bound <= T && 2 * inv_freq.numel() <= rot_dim);
+  float *wa = nullptr, *wm = nullptr;
+  TORCH_CHECK(nparts >= 1 && row_base >= 0 && row_base + rows_bound <= T);
+  if (nparts > 1) {
+    TORCH_CHECK(part_keys > 0 && part_keys % 32 == 0 && ws_acc.has_value() && ws_ml.has_value());
+    TORCH_CHECK(ws_acc->scalar_type() == at::kFloat && ws_acc->is_contiguous() &&
+                ws_acc->numel() >= nparts * heads * rows_bound * kv_rank && kv_rank % 4 == 0);
+    TORCH_CHECK(ws_ml->scalar_type() == at::kFloat && ws_ml->is_contiguous() &&
+                ws_ml->numel() >= nparts * heads * rows_bound * 2);
+    wa = ws_acc->data_ptr<float>();
+    wm = ws_ml->data_ptr<float>();
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
+  if (fill_qc)
+    hipserve::launch_latent_q_cat(qc.data_ptr(), q_abs.data_ptr<float>(), q.data_ptr(), positions.data_ptr<long>(),
+                                  inv_freq.data_ptr<float>(), inv_freq.numel(), T, heads, dim, rot_dim, kv_rank,
+                                  cur_stream());
+  hipserve::launch_latent_attention_mfma(o_lat.data_ptr(), qc.data_ptr(), proj.data_ptr(), proj.stride(0),
+                                         cache.data_ptr(), cache.size(1), seq_cu.data_ptr<int>(),
+                                         seq_ctx.data_ptr<int>(), seq_bt.data_ptr<int>(), seq_bt.size(1), seq0, seq1,
+                                         rows_bound, T, heads, rot_dim, kv_rank, gate_off, (float)scale, window,
+                                         nparts, part_keys, wa, wm, row_base, cur_stream());
+}
+
+bool latent_attention_mfma_ok(int64_t kv_rank, int64_t rot_dim) {
+  return hipserve::latent_attention_mfma_ok(kv_rank, rot_dim);
+}
+
 void mingru_scan(at::Tensor& y, at::Tensor& state, const at::Tensor& proj, const at::Tensor& b_z,
                  const at::Tensor& b_x, const at::Tensor& seq_cu, const at::Tensor& seq_ctx,
                  const at::Tensor& seq_state, int64_t max_q) {
@@ -161,6 +212,11 @@ TORCH_LIBRARY(hipserve_seq, m) {
   m.def("latent_attention(Tensor(a!) o_lat, Tensor q_abs, Tensor q, Tensor proj, Tensor cache, Tensor seq_cu, "
         "Tensor seq_ctx, Tensor seq_bt, int seq0, int seq1, int rows_bound, int tq, Tensor inv_freq, int heads, "
         "int dim, int rot_dim, int kv_rank, int gate_off, float scale, int window) -> ()");
+  m.def("latent_attention_mfma(Tensor(a!) o_lat, Tensor(b!) qc, Tensor q_abs, Tensor q, Tensor proj, Tensor positions, "
+        "Tensor cache, Tensor seq_cu, Tensor seq_ctx, Tensor seq_bt, int seq0, int seq1, int rows_bound, "
+        "Tensor inv_freq, int heads, int dim, int rot_dim, int kv_rank, int gate_off, float scale, int window, "
+        "int nparts, int part_keys, Tensor(c!)? ws_acc, Tensor(d!)? ws_ml, int row_base, bool fill_qc) -> ()");
+  m.def("latent_attention_mfma_ok(int kv_rank, int rot_dim) -> bool", &latent_attention_mfma_ok);
   m.def("mingru_scan(Tensor(a!) y, Tensor(b!) state, Tensor proj, Tensor b_z, Tensor b_x, Tensor seq_cu, "
         "Tensor seq_ctx, Tensor seq_state, int max_q) -> ()");
   m.def("moe_align(Tensor ids, int E, int tile, Tensor(a!) slots, Tensor(b!) tile_expert, Tensor(c!) pair_slot) -> ()");
@@ -172,6 +228,7 @@ TORCH_LIBRARY_IMPL(hipserve_seq, CUDA, m) {
   m.impl("scaled_add_group_rmsnorm", &scaled_add_group_rmsnorm);
   m.impl("latent_prepare", &latent_prepare);
   m.impl("latent_attention", &latent_attention);
+  m.impl("latent_attention_mfma", &latent_attention_mfma);
   m.impl("mingru_scan", &mingru_scan);
   m.impl("moe_align", &moe_align);
   m.impl("expert_gemm", &expert_gemm);

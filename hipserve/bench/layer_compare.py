@@ -1,0 +1,113 @@
+"""``bench.py --layer-compare``: prefill and decode throughput of the Kesirax layer-list
+decoder at sizes that resemble a real model's layers, beside the closest existing family
+(Mixtral-style: sliding-window attention + MoE feed-forward) at equal size. Random-init
+weights, synthetic prompts, a few layers of each (the per-layer cost is what is compared).
+
+Per size and model, through the engine's own scheduler and step function:
+  prefill tok/s  = batch x prompt_len / time of the steps that compute the prompts
+  decode tok/s   = batch x new_tokens / time of the decode steps that follow
+One JSON line per (size, model) and a last line with the ratios.
+"""
+from __future__ import annotations
+
+import json
+import time
+
+SIZES = {
+    # name: width, heads, window, experts, top, ff, gru width, vocab
+    "w1024": dict(width=1024, heads=8, window=512, experts=8, top=2, ff=512, gru=2048, vocab=32000),
+    "w2048": dict(width=2048, heads=16, window=1024, experts=16, top=2, ff=1024, gru=4096, vocab=32000),
+    "w4096": dict(width=4096, heads=32, window=1024, experts=8, top=2, ff=2048, gru=8192, vocab=32000),
+}
+
+
+def kesirax_config(name, s):
+    from ..config import HybridConfig, HybridLayerSpec, LatentAttentionSpec, MinGRUSpec, TableMoESpec
+
+    attn = LatentAttentionSpec(heads=s["heads"], dim=128, rot_dim=64, vdim=128, q_rank=s["width"] // 2,
+                               kv_rank=512, scale=192 ** -0.5, window=s["window"], rot_base=10000.0)
+    ff = TableMoESpec(experts=s["experts"], top=s["top"], ff=s["ff"])
+    layers = tuple(HybridLayerSpec(m, ff) for m in (MinGRUSpec(s["gru"]), attn, attn, MinGRUSpec(s["gru"])))
+    return HybridConfig(name=f"kesirax-{name}", hidden_size=s["width"], vocab_size=s["vocab"], layers=layers,
+                        norm_groups=4, max_position_embeddings=16384, eos_token_id=(2,), bos_token_id=1)
+
+
+def mixtral_config(name, s):
+    from ..config import ModelConfig
+
+    return ModelConfig(name=f"mixtral-{name}", architecture="mixtral", family="mixtral", hidden_size=s["width"],
+                       num_layers=4, num_heads=s["heads"], num_kv_heads=max(1, s["heads"] // 4), head_dim=128,
+                       intermediate_size=s["ff"], vocab_size=s["vocab"], rope_theta=1e6,
+                       max_position_embeddings=16384, num_experts=s["experts"], num_experts_per_tok=s["top"],
+                       sliding_window=s["window"], layer_windows=(s["window"],) * 4, bos_token_id=1, eos_token_id=(2,))
+
+
+def measure(mcfg, batch, prompt_len, new_tokens, device="cuda", repeats=2):
+    import numpy as np
+    import torch
+
+    from ..config import EngineConfig
+    from ..engine.llm_engine import LLMEngine
+    from ..engine.request import SamplingParams
+    from ..parallel.comm import TPGroup
+
+    ecfg = EngineConfig(model=mcfg.name, load_format="dummy", device=device, max_num_seqs=max(batch, 8),
+                        max_num_batched_tokens=8192, max_model_len=prompt_len + new_tokens + 8,
+                        num_kv_blocks=(batch + 2) * (-(-(prompt_len + new_tokens + 8) // 16)) + 8,
+                        enable_prefix_caching=False)
+    tp = TPGroup(0, 1, None, torch.device("cuda", 0)) if device == "cuda" else TPGroup()
+    eng = LLMEngine(ecfg, tp=tp, model_cfg=mcfg)
+    rng = np.random.default_rng(0)
+    sp = SamplingParams(temperature=0.0, max_tokens=new_tokens + 1, ignore_eos=True)
+
+    def sync():
+        if device == "cuda":
+            torch.cuda.synchronize()
+
+    best = {"prefill": 0.0, "decode": 0.0}
+    for rep in range(repeats + 1):  # the first wave warms up
+        seqs = [eng.add_request(None, rng.integers(3, mcfg.vocab_size, prompt_len).tolist(), sp) for _ in range(batch)]
+        sync()
+        t0 = time.perf_counter()
+        while any(not s.output_token_ids or s.output_token_ids[-1] < 0 for s in seqs):
+            eng.step()
+        sync()
+        t1 = time.perf_counter()
+        while eng.has_unfinished():
+            eng.step()
+        sync()
+        t2 = time.perf_counter()
+        if rep:
+            best["prefill"] = max(best["prefill"], batch * prompt_len / (t1 - t0))
+            best["decode"] = max(best["decode"], batch * new_tokens / (t2 - t1))
+    graphs = bool(eng.runner.use_graphs)
+    eng.shutdown()
+    del eng
+    if device == "cuda":
+        torch.cuda.empty_cache()
+    return {"prefill_tok_s": round(best["prefill"], 1), "decode_tok_s": round(best["decode"], 1),
+            "decode_graphs": graphs}
+
+
+def main(args) -> int:
+    sizes = [s for s in (args.layer_sizes.split(",") if args.layer_sizes else SIZES) if s]
+    device = args.device
+    out = []
+    for name in sizes:
+        s = SIZES[name]
+        row = {"size": name, **s}
+        for label, cfg in (("kesirax", kesirax_config(name, s)), ("mixtral", mixtral_config(name, s))):
+            r = measure(cfg, args.layer_batch, args.layer_prompt, args.layer_new, device)
+            row[label] = r
+            print(json.dumps({"layer_compare": name, "model": cfg.name, "batch": args.layer_batch,
+                              "prompt_len": args.layer_prompt, "new_tokens": args.layer_new, "dtype": "bf16",
+                              "data": "synthetic", **r}), flush=True)
+        row["prefill_ratio"] = round(row["kesirax"]["prefill_tok_s"] / max(row["mixtral"]["prefill_tok_s"], 1e-9), 3)
+        row["decode_ratio"] = round(row["kesirax"]["decode_tok_s"] / max(row["mixtral"]["decode_tok_s"], 1e-9), 3)
+        out.append(row)
+    print(json.dumps({"layer_compare_summary": [{k: r[k] for k in ("size", "prefill_ratio", "decode_ratio")}
+                                                for r in out]}), flush=True)
+    if args.out:
+        with open(args.out, "w") as f:
+            json.dump(out, f, indent=1)
+    return 0

@@ -625,6 +625,7 @@ class HybridConfig:
     norm_groups: int = 1
     logit_scale: float = 1.0
     max_position_embeddings: int = 1 << 20   # rotary angles are computed, not tabulated
+    default_model_len: int = 32768            # context length served when --max-model-len is not given
     bos_token_id: int | None = None
     eos_token_id: tuple = ()
     vision: object = None

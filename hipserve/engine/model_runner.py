@@ -103,8 +103,9 @@ class ModelRunner:
                 and not getattr(model_class(mcfg), "supports_fp32", False)):
             raise ValueError("the gfx950 kernels of this model run bf16 activations; use --dtype bfloat16")
         self.ops = get_ops(self.device)
-        self.max_model_len = min(ecfg.max_model_len or mcfg.max_position_embeddings,
-                                 mcfg.max_position_embeddings)
+        # no --max-model-len: the model's position range, or its serving default when that range is open-ended
+        self.max_model_len = min(ecfg.max_model_len or getattr(mcfg, "default_model_len", 0)
+                                 or mcfg.max_position_embeddings, mcfg.max_position_embeddings)
         self.block_size = ecfg.block_size
         self.model = build_model(mcfg, tp, self.device, self.dtype, self.ops, max_pos=self.max_model_len)
         # dense-transformer start-up tuning (decode GEMM autotune, weight packing, prefill padding)
@@ -627,6 +628,7 @@ class ModelRunner:
             meta.seq_bt, meta.seq_state = self._t(inp.seq_bt), self._t(inp.seq_state)
             meta.state = self.state
             meta.max_q = int(np.max(np.diff(inp.seq_cu))) if len(inp.seq_cu) > 1 else 0
+            meta.max_ctx = int(inp.seq_ctx.max()) if len(inp.seq_ctx) else 0
         if "mm" in inp.extra:
             self._attach_mm(inp.extra["mm"], meta, len(inp.ids))
         hidden = self.model.forward(ids, meta, self.kv)
@@ -714,6 +716,10 @@ class ModelRunner:
         meta = AttnMeta(num_prefill_tokens=0, num_decode=b, positions=st["pos"][:b],
                         slot_mapping=st["slots"][:b], bt_decode=st["bt"][:b], ctx_decode=st["ctx"][:b],
                         tmp_out=self.tmp_out, tmp_ml=self.tmp_ml)
+        if self.seq_meta:  # every row is one decode sequence
+            meta.seq_cu, meta.seq_ctx, meta.seq_bt = st["cu"][:b + 1], st["ctx"][:b], st["bt"][:b]
+            meta.seq_state, meta.state = st["sslot"][:b], self.state
+            meta.max_q, meta.max_ctx = 1, self.max_model_len
         # lookahead ids: resolved inside the model's first kernel when it can
         # (embed_rmsnorm), else by the model's id select (LlamaModel.resolve_ids)
         meta.id_src = (st["src"][:b], st["tok"])
@@ -753,7 +759,7 @@ class ModelRunner:
         for _ in range(2):
             self._stage.append({
                 "h64": torch.zeros(6 * mb, dtype=torch.long).pin_memory(),
-                "h32": torch.zeros(mb * W + 4 * mb, dtype=torch.int32).pin_memory(),
+                "h32": torch.zeros(mb * W + 5 * mb, dtype=torch.int32).pin_memory(),
                 "hf": torch.zeros(5 * mb, dtype=torch.float32).pin_memory(),
                 "tok": torch.zeros(mb, dtype=torch.long).pin_memory(),
                 "lp": torch.zeros(mb, dtype=torch.float32).pin_memory(),
@@ -765,7 +771,7 @@ class ModelRunner:
         # HIPSERVE_STAGE_COPY=blit: per-buffer hipMemcpyAsync instead of the staging kernel
         self._stage_kernel = os.environ.get("HIPSERVE_STAGE_COPY", "kernel") != "blit"
         d64 = torch.zeros(6 * mb, dtype=torch.long, device=dev)
-        d32 = torch.zeros(mb * W + 4 * mb, dtype=torch.int32, device=dev)
+        d32 = torch.zeros(mb * W + 5 * mb, dtype=torch.int32, device=dev)
         df = torch.zeros(5 * mb, dtype=torch.float32, device=dev)
         st = {
             "d64": d64, "d32": d32, "df": df,
@@ -774,6 +780,9 @@ class ModelRunner:
             "bt": d32[: mb * W].view(mb, W), "ctx": d32[mb * W: mb * W + mb],
             "topk": d32[mb * W + mb: mb * W + 2 * mb],
             "pslot": d32[mb * W + 2 * mb: mb * W + 3 * mb], "nlp": d32[mb * W + 3 * mb: mb * W + 4 * mb],
+            # recurrent-state slot per row (padding rows: the scratch slot) and the rows' offsets 0..mb
+            "sslot": d32[mb * W + 4 * mb: mb * W + 5 * mb],
+            "cu": torch.arange(mb + 1, dtype=torch.int32, device=dev),
             "temp": df[0:mb], "topp": df[mb:2 * mb],
             "pres": df[2 * mb:3 * mb], "freq": df[3 * mb:4 * mb], "rep": df[4 * mb:5 * mb],
             "tok": torch.zeros(mb, dtype=torch.long, device=dev),
@@ -788,6 +797,7 @@ class ModelRunner:
         st["topp"].fill_(1.0)
         st["src"].fill_(-1)
         st["pslot"].fill_(-1)
+        st["sslot"].fill_(self.num_state_slots)
         st["rep"].fill_(1.0)
         t0 = time.time()
         # TP ranks enter the captured collectives together (the tuner and the
@@ -870,6 +880,8 @@ class ModelRunner:
         a32[o + n:o + b] = -1
         a32[o + mb:o + mb + n] = inp.nlogprobs if inp.nlogprobs is not None else 0
         a32[o + mb + n:o + mb + b] = 0
+        a32[o + 2 * mb:o + 2 * mb + n] = inp.seq_state if inp.seq_state is not None else 0
+        a32[o + 2 * mb + n:o + 2 * mb + b] = self.num_state_slots  # the scratch slot
         af = hf.numpy()
         af[0:n] = inp.temperature
         af[n:b] = 0.0

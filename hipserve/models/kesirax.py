@@ -37,7 +37,7 @@ class _Layer:
 
 class KesiraxModel:
     supports_fp32 = True        # every op of this model has a true 32-bit build
-    graph_decode = False        # decode steps run eagerly
+    graph_decode = True         # decode-only steps replay a captured hipGraph
 
     def __init__(self, cfg: HybridConfig, tp: TPGroup, device, dtype=torch.bfloat16, ops=None,
                  max_pos: int | None = None):
@@ -164,6 +164,9 @@ class KesiraxModel:
         ops, cfg = self.ops, self.cfg
         T, H = ids.shape[0], cfg.hidden_size
         state = meta.state
+        if meta.id_src is not None:  # decode lookahead: row i's id is the previous step's sample tok[src[i]]
+            src, tok = meta.id_src
+            ids = torch.where(src >= 0, tok.index_select(0, src.clamp(min=0)), ids)
         x0 = F.embedding(ids, self.embed)                 # the embedding output (model dtype)
         residual = x0.to(torch.float32, copy=True)    # never an alias of x0 (float32 models)
         h = torch.empty(T, H, device=x0.device, dtype=self.dtype)

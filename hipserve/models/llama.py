@@ -75,6 +75,7 @@ class AttnMeta:
     seq_state: torch.Tensor | None = None
     state: list | None = None
     max_q: int = 0
+    max_ctx: int = 0   # longest context of the step (host; a captured step: the model length)
 
 
 @dataclass

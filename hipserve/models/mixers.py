@@ -27,7 +27,8 @@ import torch.nn.functional as F
 
 from ..config import LatentAttentionSpec, MinGRUSpec, TableMoESpec
 
-MOE_TILE = 32  # slots per expert tile of the expert GEMMs
+MOE_TILE = 32        # slots per expert tile of the expert GEMMs ...
+MOE_TILE_LARGE = 64  # ... when every expert has several tiles' worth of rows on average
 
 
 def _mm32(x: torch.Tensor, w_t: torch.Tensor) -> torch.Tensor:
@@ -162,7 +163,8 @@ class TableMoE:
         s, ops = self.spec, self.ops
         T, dev = h.shape[0], h.device
         experts = self.table.index_select(0, ids).reshape(-1)          # [T * top]
-        P, tile = T * s.top, MOE_TILE
+        P = T * s.top
+        tile = MOE_TILE_LARGE if P >= 4 * MOE_TILE_LARGE * s.experts else MOE_TILE
         cap = -(-(P + s.experts * (tile - 1)) // tile) * tile
         slots = torch.empty(cap, dtype=torch.int32, device=dev)
         tile_expert = torch.empty(cap // tile, dtype=torch.int32, device=dev)

@@ -190,15 +190,41 @@ class KernelOps:
                                  rot_dim, eps)
 
     LATENT_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x up to 4 heads = 16 waves)
+    # bf16 runs the MFMA kernel (HIPSERVE_LATENT_MFMA=0: the generic kernel, as fp32 does)
+    LATENT_MFMA = os.environ.get("HIPSERVE_LATENT_MFMA", "1") != "0"
+    LATENT_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32)
 
     def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
                          gate_off, scale, window):
         """Prompt portions (the step's first sequences) run several tokens per workgroup, decode
-        rows one token x up to 16 heads; both on the same kernel."""
+        rows one token per workgroup."""
         nseq = meta.seq_ctx.shape[0]
-        npf = nseq - meta.num_decode
-        for s0, s1, rows, tq in ((0, npf, meta.num_prefill_tokens, self.LATENT_PREFILL_TQ),
-                                 (npf, nseq, meta.num_decode, 1)):
+        nd = meta.num_decode
+        npf, Tp = nseq - nd, meta.num_prefill_tokens
+        if (q.dtype == torch.bfloat16 and self.LATENT_MFMA and self._seq.latent_attention_mfma_ok(kv_rank, rot_dim)):
+            # bf16: the matrix-core kernel; decode rows split their keys into runs merged by a reduce kernel
+            qc = torch.empty(heads, q.shape[0], kv_rank + rot_dim, device=q.device, dtype=q.dtype)
+            fill = True
+            if npf:
+                self._seq.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
+                                                meta.seq_ctx, meta.seq_bt, 0, npf, Tp, inv_freq, heads, dim, rot_dim,
+                                                kv_rank, gate_off, scale, window, 1, 0, None, None, 0, fill)
+                fill = False
+            if nd:
+                span = min(window, meta.max_ctx or window) if window > 0 else meta.max_ctx
+                part = self.LATENT_DECODE_RUN
+                while -(-span // part) > 64:
+                    part *= 2
+                nparts = max(1, -(-span // part))
+                ws_acc = ws_ml = None
+                if nparts > 1:
+                    ws_acc = torch.empty(nparts, heads, nd, kv_rank, device=q.device, dtype=torch.float32)
+                    ws_ml = torch.empty(nparts, heads, nd, 2, device=q.device, dtype=torch.float32)
+                self._seq.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
+                                                meta.seq_ctx, meta.seq_bt, npf, nseq, nd, inv_freq, heads, dim, rot_dim,
+                                                kv_rank, gate_off, scale, window, nparts, part, ws_acc, ws_ml, Tp, fill)
+            return
+        for s0, s1, rows, tq in ((0, npf, Tp, self.LATENT_PREFILL_TQ), (npf, nseq, nd, 1)):
             if s1 > s0:
                 self._seq.latent_attention(o_lat, q_abs, q, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt,
                                            s0, s1, rows, tq, inv_freq, heads, dim, rot_dim, kv_rank, gate_off,

@@ -273,10 +273,10 @@ def test_far_key_across_pages(tmp_path, target):
     """A sharp softmax (large scale) and a window longer than the prompt: most of the weight of a
     late query sits on single keys hundreds of tokens back, in other pages of the cache. (bf16 runs a
     less sharp softmax: at scale 6 the rounding of the scores alone moves the weights.)"""
-    sc = 6.0 if target[1] == "float32" else 2.0
+    sc, gain = (6.0, 1.5) if target[1] == "float32" else (1.0, 1.0)
     cfg = O.make_config([O.attn_layer(window=1000, scale=sc, heads=2), O.attn_layer(window=0, scale=sc, heads=2)],
                         groups=1)
-    W = O.make_weights(cfg, seed=15, gain=1.5)
+    W = O.make_weights(cfg, seed=15, gain=gain)
     toks = tokens(330, cfg["vocab"], 4)
     ref = O.forward(cfg, W, toks)
     near = O.make_config([O.attn_layer(window=200, scale=sc, heads=2), O.attn_layer(window=200, scale=sc, heads=2)],
