@@ -81,6 +81,7 @@ def parse():
                     help="instead of the headline benchmark: prefill / decode tok/s of the Kesirax decoder "
                          "beside a Mixtral-style model of equal size (hipserve/bench/layer_compare.py)")
     ap.add_argument("--layer-sizes", default="", help="with --layer-compare: sizes, comma separated (default: all)")
+    ap.add_argument("--layer-models", default="", help="with --layer-compare: kesirax, mixtral or both (default)")
     ap.add_argument("--layer-batch", type=int, default=16)
     ap.add_argument("--layer-prompt", type=int, default=2048)
     ap.add_argument("--layer-new", type=int, default=64)

@@ -173,6 +173,8 @@ constexpr int PG_EPI_STORE = 0, PG_EPI_ADD = 1, PG_EPI_GLU = 2, PG_EPI_GEGLU = 3
 //   PW_EPI_STORE / PW_EPI_ADD as PG_*; PW_EPI_GLU / PW_EPI_GEGLU: W packed with glu = true
 //   (merged [gate; up], N = 2I, I % 64 == 0), C = act [M, I]
 constexpr int PW_EPI_STORE = 0, PW_EPI_ADD = 1, PW_EPI_GLU = 2, PW_EPI_GEGLU = 3;
+// PW_EPI_RELU2: as STORE with C = bf16(max(acc, 0)^2) (the squared-ReLU experts of the table-routed MoE)
+constexpr int PW_EPI_RELU2 = 4;
 // grid_req <= 0: persistent (one workgroup per CU walking the tiles), else that many workgroups.
 // rw: weight register sets in flight (2 or 4 32-deep slots ahead; 5 = 4 with each reload
 // issued one MFMA group later).

@@ -39,6 +39,7 @@
 //                 rows): gate rg and up rg + 4 sit in the same lane, so
 //                 act[m, 64 t + 16 rg + 4 (l >> 4) + j] = silu(gate) * up in registers
 //   PW_EPI_GEGLU  as GLU with tanh-GELU (Gemma)
+//   PW_EPI_RELU2  C = bf16(max(acc, 0)^2): the table-routed experts' squared ReLU
 #include "hipserve/common.h"
 #include "hipserve/kernels.h"
 
@@ -305,6 +306,13 @@ __global__ __launch_bounds__(PW_T) __attribute__((amdgpu_waves_per_eu(1, 1))) vo
             } else {  // bias added to the fp32 accumulator, one rounding
 #pragma unroll
               for (int j = 0; j < 4; ++j) o[j] = acc[rg][i][j] + bv[j];
+              if constexpr (EPI == PW_EPI_RELU2) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  const float r = fmaxf(o[j], 0.f);
+                  o[j] = r * r;
+                }
+              }
             }
             *dst = uint2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
           }
@@ -374,6 +382,7 @@ bool launch_prefill_gemm_packed(int epi, void* C, long ldc, const void* X, long 
     case PW_EPI_ADD: PW_LAUNCH(WM_, PW_EPI_ADD); return true;     \
     case PW_EPI_GLU: PW_LAUNCH(WM_, PW_EPI_GLU); return true;     \
     case PW_EPI_GEGLU: PW_LAUNCH(WM_, PW_EPI_GEGLU); return true; \
+    case PW_EPI_RELU2: PW_LAUNCH(WM_, PW_EPI_RELU2); return true; \
     default: return false;                                    \
   }
   if (wm == 1) {

@@ -102,20 +102,26 @@ __global__ __launch_bounds__(256) void expert_gemm_mfma_kernel(
 #pragma unroll
     for (int st = 0; st < ST; ++st) acc[nt][st] = f32x4{0.f, 0.f, 0.f, 0.f};
   const u16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 2
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const bool in = k0 + 8 * g < K;
-    u16x8 a[2], b[ST];
+  constexpr int kU = 4;  // k steps whose operand loads are in flight together
+  for (int k0 = 0; k0 < K; k0 += 32 * kU) {
+    u16x8 a[kU][2], b[kU][ST];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) a[nt] = in ? *reinterpret_cast<const u16x8*>(wr[nt] + k0) : zero;
+    for (int u = 0; u < kU; ++u) {
+      const int k = k0 + 32 * u;
+      const bool in = k + 8 * g < K;
 #pragma unroll
-    for (int st = 0; st < ST; ++st) b[st] = (in && live[st]) ? *reinterpret_cast<const u16x8*>(xr[st] + k0) : zero;
+      for (int nt = 0; nt < 2; ++nt) a[u][nt] = in ? *reinterpret_cast<const u16x8*>(wr[nt] + k) : zero;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+      for (int st = 0; st < ST; ++st) b[u][st] = (in && live[st]) ? *reinterpret_cast<const u16x8*>(xr[st] + k) : zero;
+    }
 #pragma unroll
-      for (int st = 0; st < ST; ++st)
-        acc[nt][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[nt]),
-                                                              __builtin_bit_cast(bf16x8, b[st]), acc[nt][st], 0, 0, 0);
+    for (int u = 0; u < kU; ++u)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int st = 0; st < ST; ++st)
+          acc[nt][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u][nt]),
+                                                                __builtin_bit_cast(bf16x8, b[u][st]), acc[nt][st], 0, 0, 0);
   }
   // lane (c, g): columns n0 + 16 nt + 4 g .. + 3 of slot 16 st + c
 #pragma unroll

@@ -134,18 +134,29 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   const bool sact = srt < ntok && srh < nh;
   const int spos = p_first + srt;
   const int s_lo = window > 0 ? max(0, spos - window + 1) : 0;
+  constexpr int kFill = (KS * 4 + 7) / 8;
+  u16x8 fv[kFill];
+  // the thread's part of a tile, all loads in flight together; zero past Dk and past the last key
+  auto fetch = [&](int j0) {
+    const int j = j0 + fkey;
+    const bool in = j <= hi;
+    const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dk : 0;
+#pragma unroll
+    for (int i = 0; i < kFill; ++i) {
+      const int ch = fk + 8 * i;
+      fv[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (in && ch < chunks) fv[i] = *reinterpret_cast<const u16x8*>(cache + kr + 8 * ch);
+    }
+  };
+  if (lo <= hi) fetch(lo);
   for (int j0 = lo; j0 <= hi; j0 += kKeys) {
     __syncthreads();  // the previous tile's reads of the K tile (P . V) are done
-    {
-      const int j = j0 + fkey;
-      const bool in = j <= hi;
-      const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dk : 0;
-      for (int ch = fk; ch < KS * 4; ch += 8) {  // zero past Dk and past the last key
-        u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (in && ch < chunks) v = *reinterpret_cast<const u16x8*>(cache + kr + 8 * ch);
-        *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = v;
-      }
+#pragma unroll
+    for (int i = 0; i < kFill; ++i) {
+      const int ch = fk + 8 * i;
+      if (ch < KS * 4) *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = fv[i];
     }
+    if (j0 + kKeys <= hi) fetch(j0 + kKeys);  // the next tile travels while this one is computed
     __syncthreads();
     // 1. S^T tiles: a = keys (16 per tile), b = this wave's 16 query rows
     f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -182,7 +193,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
       u16x8 pk;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = (v[e] > -INFINITY) ? expf(v[e] - mn) : 0.f;
+        const float p = (v[e] > -INFINITY) ? __expf(v[e] - mn) : 0.f;  // rounded to bf16 right below
         const unsigned short pb = f32_to_bf16(p);
         pk[e] = pb;
         sum += bf16_to_f32(pb);  // the sum of the weights that are actually multiplied
@@ -202,10 +213,18 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     //    (g, e) is key 4 e + g, read column-wise from the row-major K tile
     bf16x8 pb[4];
     float al[4];
+    bool rescale = false;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       pb[mt] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(p_lds + (16 * mt + c) * kPLd + 8 * g));
       al[mt] = alpha[16 * mt + c];
+      rescale |= al[mt] != 1.f;
+    }
+    if (__any(rescale)) {  // the running maxima settle after a few tiles: most tiles skip this
+#pragma unroll
+      for (int j = 0; j < NPW; ++j)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[mt][j] *= al[mt];
     }
 #pragma unroll
     for (int j = 0; j < NPW; ++j) {
@@ -215,10 +234,8 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) a[e] = kt[(4 * e + g) * kLd + 16 * nt + c];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-          acc[mt][j] *= al[mt];
+        for (int mt = 0; mt < 4; ++mt)
           acc[mt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb[mt], acc[mt][j], 0, 0, 0);
-        }
       }
     }
   }

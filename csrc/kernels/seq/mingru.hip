@@ -14,15 +14,6 @@ namespace {
 constexpr int kMaxWaves = 16;
 
 template <typename T>
-HS_DEVICE void gate_cand(const T* __restrict__ proj, long row, int width, int c, float bz, float bx, float& z,
-                         float& cand) {
-  const long base = row * 3 * width;
-  z = sigmoid_f(ldf<T>(proj, base + c) + bz);
-  const float u = ldf<T>(proj, base + width + c) + bx;
-  cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
-}
-
-template <typename T>
 __global__ __launch_bounds__(64 * kMaxWaves) void mingru_scan_kernel(
     T* __restrict__ y, float* __restrict__ state, const T* __restrict__ proj, const float* __restrict__ b_z,
     const float* __restrict__ b_x, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx,
@@ -38,12 +29,28 @@ __global__ __launch_bounds__(64 * kMaxWaves) void mingru_scan_kernel(
   const float bz = b_z[cc], bx = b_x[cc];
   const int per = (n + nw - 1) / nw;
   const int a = min(wave * per, n), b = min(a + per, n);
+  // rows go through in blocks of kB: the block's loads are issued together, then the serial update
+  constexpr int kB = 8;
+  const long ld = 3L * width;
   float A = 1.f, B = 0.f;
-  for (int t = a; t < b; ++t) {
-    float z, cand;
-    gate_cand<T>(proj, r0 + t, width, cc, bz, bx, z, cand);
-    A *= 1.f - z;
-    B = (1.f - z) * B + z * cand;
+  for (int t0 = a; t0 < b; t0 += kB) {
+    float zp[kB], xp[kB];
+#pragma unroll
+    for (int i = 0; i < kB; ++i) {
+      const long base = (long)(r0 + min(t0 + i, b - 1)) * ld;
+      zp[i] = ldf<T>(proj, base + cc);
+      xp[i] = ldf<T>(proj, base + width + cc);
+    }
+#pragma unroll
+    for (int i = 0; i < kB; ++i) {
+      if (t0 + i < b) {
+        const float z = sigmoid_f(zp[i] + bz);
+        const float u = xp[i] + bx;
+        const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+        A *= 1.f - z;
+        B = (1.f - z) * B + z * cand;
+      }
+    }
   }
   sa[wave][lane] = A;
   sb[wave][lane] = B;
@@ -52,12 +59,25 @@ __global__ __launch_bounds__(64 * kMaxWaves) void mingru_scan_kernel(
   float S = (seq_ctx[s] - n > 0) ? state[slot] : 0.f;
   __syncthreads();
   for (int k = 0; k < wave; ++k) S = sa[k][lane] * S + sb[k][lane];
-  for (int t = a; t < b; ++t) {
-    float z, cand;
-    gate_cand<T>(proj, r0 + t, width, cc, bz, bx, z, cand);
-    S = (1.f - z) * S + z * cand;
-    const float g = ldf<T>(proj, (long)(r0 + t) * 3 * width + 2 * width + cc);
-    if (live) stf<T>(y, (long)(r0 + t) * width + c, S * (g * sigmoid_f(g)));
+  for (int t0 = a; t0 < b; t0 += kB) {
+    float zp[kB], xp[kB], gp[kB];
+#pragma unroll
+    for (int i = 0; i < kB; ++i) {
+      const long base = (long)(r0 + min(t0 + i, b - 1)) * ld;
+      zp[i] = ldf<T>(proj, base + cc);
+      xp[i] = ldf<T>(proj, base + width + cc);
+      gp[i] = ldf<T>(proj, base + 2 * width + cc);
+    }
+#pragma unroll
+    for (int i = 0; i < kB; ++i) {
+      if (t0 + i < b) {
+        const float z = sigmoid_f(zp[i] + bz);
+        const float u = xp[i] + bx;
+        const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+        S = (1.f - z) * S + z * cand;
+        if (live) stf<T>(y, (long)(r0 + t0 + i) * width + c, S * (gp[i] * sigmoid_f(gp[i])));
+      }
+    }
   }
   // the wave that holds the last row leaves the state (empty trailing segments keep S = chained value)
   if (live && wave == nw - 1) state[slot] = S;

@@ -848,7 +848,7 @@ void prefill_gemm_packed_grouped(at::Tensor& out, const at::Tensor& x, const at:
   TORCH_CHECK(M % (128 * wm) == 0 && tile_expert.numel() >= M / (128 * wm), "prefill_gemm_packed_grouped: tiles");
   TORCH_CHECK(tile_expert.scalar_type() == at::kInt && num_tiles.scalar_type() == at::kInt, "int32 tile tables");
   const bool glu = epi == 2 || epi == 3;
-  TORCH_CHECK(epi == 0 || glu, "prefill_gemm_packed_grouped: store or glu epilogue");
+  TORCH_CHECK(epi == 0 || epi == 4 || glu, "prefill_gemm_packed_grouped: store, squared-ReLU or glu epilogue");
   TORCH_CHECK(out.size(0) == M && out.size(1) == (glu ? N / 2 : N), "prefill_gemm_packed_grouped: out shape");
   c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
   hipserve::PwGroup grp{tile_expert.data_ptr<int>(), num_tiles.data_ptr<int>(), (long)wp.size(1)};

@@ -96,16 +96,22 @@ def main(args) -> int:
     for name in sizes:
         s = SIZES[name]
         row = {"size": name, **s}
+        models = [m for m in (args.layer_models or "kesirax,mixtral").split(",") if m]
         for label, cfg in (("kesirax", kesirax_config(name, s)), ("mixtral", mixtral_config(name, s))):
+            if label not in models:
+                continue
             r = measure(cfg, args.layer_batch, args.layer_prompt, args.layer_new, device)
             row[label] = r
             print(json.dumps({"layer_compare": name, "model": cfg.name, "batch": args.layer_batch,
                               "prompt_len": args.layer_prompt, "new_tokens": args.layer_new, "dtype": "bf16",
                               "data": "synthetic", **r}), flush=True)
+        if "kesirax" not in row or "mixtral" not in row:
+            out.append(row)
+            continue
         row["prefill_ratio"] = round(row["kesirax"]["prefill_tok_s"] / max(row["mixtral"]["prefill_tok_s"], 1e-9), 3)
         row["decode_ratio"] = round(row["kesirax"]["decode_tok_s"] / max(row["mixtral"]["decode_tok_s"], 1e-9), 3)
         out.append(row)
-    print(json.dumps({"layer_compare_summary": [{k: r[k] for k in ("size", "prefill_ratio", "decode_ratio")}
+    print(json.dumps({"layer_compare_summary": [{k: r.get(k) for k in ("size", "prefill_ratio", "decode_ratio")}
                                                 for r in out]}), flush=True)
     if args.out:
         with open(args.out, "w") as f:

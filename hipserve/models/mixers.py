@@ -29,6 +29,10 @@ from ..config import LatentAttentionSpec, MinGRUSpec, TableMoESpec
 
 MOE_TILE = 32        # slots per expert tile of the expert GEMMs ...
 MOE_TILE_LARGE = 64  # ... when every expert has several tiles' worth of rows on average
+# bf16 batches with at least this many (token, expert) pairs per expert run the packed-layout grouped
+# GEMM of the dense families' MoE prefill (prefill_gemm_packed.hip: 128-row tiles, X through LDS, the
+# weights pre-shuffled into MFMA operand order) with the squared ReLU in its epilogue
+MOE_PACKED_MIN_PAIRS_PER_EXPERT = 256
 
 
 def _mm32(x: torch.Tensor, w_t: torch.Tensor) -> torch.Tensor:
@@ -143,6 +147,7 @@ class TableMoE:
         self.table = None   # int32 [vocab, top]
         self.w_up = None    # [E, ff, hidden]
         self.w_down = None  # [E, hidden, ff]
+        self.packed = None  # (up, down) in the packed grouped-GEMM layout, made at the first large batch
 
     def load(self, get, prefix: str):
         dt, dev, E = self.dtype, self.device, self.spec.experts
@@ -164,6 +169,8 @@ class TableMoE:
         T, dev = h.shape[0], h.device
         experts = self.table.index_select(0, ids).reshape(-1)          # [T * top]
         P = T * s.top
+        if self._packed_ok(h, P):
+            return self._forward_packed(h, experts, P)
         tile = MOE_TILE_LARGE if P >= 4 * MOE_TILE_LARGE * s.experts else MOE_TILE
         cap = -(-(P + s.experts * (tile - 1)) // tile) * tile
         slots = torch.empty(cap, dtype=torch.int32, device=dev)
@@ -174,4 +181,38 @@ class TableMoE:
         ops.expert_gemm(act, h, self.w_up, slots, tile_expert, tile, s.top, True)
         y = torch.empty(cap, self.hidden, device=dev, dtype=h.dtype)
         ops.expert_gemm(y, act, self.w_down, slots, tile_expert, tile, 0, False)
+        return y, pair_slot
+
+    def _packed_ok(self, h: torch.Tensor, P: int) -> bool:
+        s = self.spec
+        return (getattr(self.ops, "name", "") == "hip" and h.dtype == torch.bfloat16 and s.experts <= 128
+                and self.hidden % 256 == 0 and s.ff % 256 == 0
+                and P >= MOE_PACKED_MIN_PAIRS_PER_EXPERT * s.experts and not torch.cuda.is_current_stream_capturing())
+
+    def _forward_packed(self, h: torch.Tensor, experts: torch.Tensor, P: int):
+        """Large bf16 batches: the experts as two launches of the packed-layout grouped GEMM (token rows
+        gathered through the slot table inside the first one, squared ReLU in its epilogue)."""
+        from ..ops import gemm
+
+        s, dev = self.spec, h.device
+        op = self.ops._op  # the core kernel library
+        E, H, ff = s.experts, self.hidden, s.ff
+        if self.packed is None:
+            pu = torch.empty(E, -(-ff // 128) * 128 * H, dtype=h.dtype, device=dev)
+            pd = torch.empty(E, -(-H // 128) * 128 * ff, dtype=h.dtype, device=dev)
+            op.pack_decode_weight(pu, self.w_up, False)
+            op.pack_decode_weight(pd, self.w_down, False)
+            self.packed = (pu, pd)
+        tile = 128 * gemm.PW_WM
+        cap = -(-(P + E * (tile - 1)) // tile) * tile
+        slots = torch.empty(cap, dtype=torch.int32, device=dev)
+        tile_expert = torch.empty(cap // tile, dtype=torch.int32, device=dev)
+        ntiles = torch.empty(1, dtype=torch.int32, device=dev)
+        pair_slot = torch.empty(P, dtype=torch.int32, device=dev)
+        op.moe_align(experts, E, tile, slots, tile_expert, ntiles, pair_slot, None)
+        pu, pd = self.packed
+        act = torch.empty(cap, ff, dtype=h.dtype, device=dev)
+        op.prefill_gemm_packed_grouped(act, h, pu, ff, 4, tile_expert, ntiles, gemm.PW_WM, gemm.PW_RW, slots, s.top)
+        y = torch.empty(cap, H, dtype=h.dtype, device=dev)
+        op.prefill_gemm_packed_grouped(y, act, pd, H, 0, tile_expert, ntiles, gemm.PW_WM, gemm.PW_RW)
         return y, pair_slot

@@ -334,3 +334,27 @@ def test_greedy_generation_through_the_scheduler(tmp_path, target):
             row = lg[len(p) + k - 1]
             assert row[t] >= row.max() - slack, (k, t, int(row.argmax()))
     assert eng.states.num_free() == 4 and eng.blocks.num_free() == eng.blocks.num_blocks
+
+
+@pytest.mark.gpu
+def test_table_moe_large_batch_gpu():
+    """bf16 batches with many rows per expert take the packed-layout grouped GEMM (squared ReLU in its
+    epilogue); same result as the plain experts."""
+    from hipserve.models import mixers
+
+    dev = torch.device("cuda")
+    f = O.moe(experts=2, top=1, ff=256)
+    cfg = O.make_config([O.gru_layer(mlp=f)], width=256, vocab=64, groups=1)
+    W = O.make_weights(cfg, seed=21)
+    T = 640
+    toks = tokens(T, 64, 9)
+    h = torch.randn(T, 256, generator=torch.Generator().manual_seed(5)).bfloat16().float()
+    want = O.table_moe(h, toks, W, "l0.mlp.", f)
+    moe = TableMoE(HybridConfig.from_dict(cfg).layers[0].mlp, 256, 64, dev, torch.bfloat16, get_ops(dev))
+    moe.load(lambda k: W[k], "l0.mlp.")
+    assert moe._packed_ok(h.to(dev, torch.bfloat16), T)
+    y, pair_slot = moe.forward(h.to(dev, torch.bfloat16), torch.tensor(toks, device=dev))
+    assert moe.packed is not None
+    got = y.float().index_select(0, pair_slot.long())
+    assert rel_err(got, want) < TOL["bfloat16"]
+    assert mixers.MOE_PACKED_MIN_PAIRS_PER_EXPERT * 2 <= T
