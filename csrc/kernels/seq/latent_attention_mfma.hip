@@ -92,6 +92,8 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   float* m_run = alpha + kRows;                                                    // [64]
   float* l_run = m_run + kRows;                                                    // [64]
   int s, tok0;
+  // (workgroups are dealt to the XCDs round-robin; giving each XCD a contiguous run of token tiles was
+  // measured slower, 1188 vs 1013 us at 8192 tokens x 16 heads: the causal start makes the runs unequal)
   if (!find_tile64(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) return;
   const int Dk = kv_rank + rot_dim;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

@@ -192,7 +192,7 @@ class KernelOps:
     LATENT_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x up to 4 heads = 16 waves)
     # bf16 runs the MFMA kernel (HIPSERVE_LATENT_MFMA=0: the generic kernel, as fp32 does)
     LATENT_MFMA = os.environ.get("HIPSERVE_LATENT_MFMA", "1") != "0"
-    LATENT_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32)
+    LATENT_DECODE_RUN = 64   # keys per run of a decode row (a multiple of 32)
 
     def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
                          gate_off, scale, window):
