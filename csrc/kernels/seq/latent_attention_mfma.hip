@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void latent_q_cat_kernel(unsigned short* __res
   }
 }
 
-constexpr int kRows = 64;   // (token, head) rows per workgroup
+// (token, head) rows per workgroup = 16 x its waves NW (4: 64 rows)
 constexpr int kKeys = 32;   // keys per tile
 constexpr int kPLd = 40;    // P tile row stride (elements): 16-byte aligned rows, padded
 
@@ -76,14 +76,15 @@ template <int KS> struct KtLd { static constexpr int v = KS * 32 + ((KS & 1) ? 4
 // KS: 32-dim steps of a cache row (Dk <= 32 KS); NPW: 16-dim output tiles per wave (kv_rank <= 64 NPW).
 // grid.z > 1 splits the keys of a row into runs of part_keys; the runs' unnormalised outputs and
 // (max, sum) go to ws_acc / ws_ml for latent_attention_reduce (decode rows: many keys, few rows).
-template <int KS, int NPW>
-__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+template <int KS, int NPW, int NW>
+__global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
     unsigned short* __restrict__ o_lat, const unsigned short* __restrict__ qc, const unsigned short* __restrict__ proj,
     long proj_ld, const unsigned short* __restrict__ cache, int block_size, const int* __restrict__ seq_cu,
     const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
     int T_rows, int heads, int rot_dim, int kv_rank, int gate_off, float scale, int window, int part_keys,
     float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows) {
   constexpr int kLd = KtLd<KS>::v;
+  constexpr int kRows = 16 * NW, kThreads = 64 * NW, kFT = kThreads / kKeys;  // kFT threads fill one key's row
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned short* kt = reinterpret_cast<unsigned short*>(smem);                    // [32][kLd] bf16 cache rows
   float* s_lds = reinterpret_cast<float*>(smem + kKeys * kLd * 2);                 // [64][32] fp32 scores
@@ -121,22 +122,22 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
   }
   if (tid < kRows) { m_run[tid] = -INFINITY; l_run[tid] = 0.f; }
-  f32x4 acc[4][NPW];
+  f32x4 acc[NW][NPW];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int mt = 0; mt < NW; ++mt)
 #pragma unroll
     for (int j = 0; j < NPW; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int ntiles_dv = (kv_rank + 15) / 16;
   const int chunks = Dk / 8;  // 16-byte chunks of a cache row
-  // tile fill: 8 threads per key, each its key's chunks fk, fk + 8, ...
-  const int fkey = tid >> 3, fk = tid & 7;
+  // tile fill: kFT threads per key, each its key's chunks fk, fk + kFT, ...
+  const int fkey = tid / kFT, fk = tid % kFT;
   // softmax: 4 threads per row; thread `part` owns the keys 4 e + part (e = 0..7) of the tile
   const int sr = tid >> 2, part = tid & 3;
   const int srt = sr / hc, srh = sr % hc;
   const bool sact = srt < ntok && srh < nh;
   const int spos = p_first + srt;
   const int s_lo = window > 0 ? max(0, spos - window + 1) : 0;
-  constexpr int kFill = (KS * 4 + 7) / 8;
+  constexpr int kFill = (KS * 4 + kFT - 1) / kFT;
   u16x8 fv[kFill];
   // the thread's part of a tile, all loads in flight together; zero past Dk and past the last key
   auto fetch = [&](int j0) {
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dk : 0;
 #pragma unroll
     for (int i = 0; i < kFill; ++i) {
-      const int ch = fk + 8 * i;
+      const int ch = fk + kFT * i;
       fv[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
       if (in && ch < chunks) fv[i] = *reinterpret_cast<const u16x8*>(cache + kr + 8 * ch);
     }
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     __syncthreads();  // the previous tile's reads of the K tile (P . V) are done
 #pragma unroll
     for (int i = 0; i < kFill; ++i) {
-      const int ch = fk + 8 * i;
+      const int ch = fk + kFT * i;
       if (ch < KS * 4) *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = fv[i];
     }
     if (j0 + kKeys <= hi) fetch(j0 + kKeys);  // the next tile travels while this one is computed
@@ -213,11 +214,11 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     __syncthreads();
     // 3. acc[rows][dims] = acc * alpha + V^T . P^T: a = 16 latent dims, b = 16 rows; the MFMA's k slot
     //    (g, e) is key 4 e + g, read column-wise from the row-major K tile
-    bf16x8 pb[4];
-    float al[4];
+    bf16x8 pb[NW];
+    float al[NW];
     bool rescale = false;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < NW; ++mt) {
       pb[mt] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(p_lds + (16 * mt + c) * kPLd + 8 * g));
       al[mt] = alpha[16 * mt + c];
       rescale |= al[mt] != 1.f;
@@ -226,17 +227,17 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
       for (int j = 0; j < NPW; ++j)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[mt][j] *= al[mt];
+        for (int mt = 0; mt < NW; ++mt) acc[mt][j] *= al[mt];
     }
 #pragma unroll
     for (int j = 0; j < NPW; ++j) {
-      const int nt = wave + 4 * j;
+      const int nt = wave + NW * j;
       if (nt < ntiles_dv) {
         u16x8 a;
 #pragma unroll
         for (int e = 0; e < 8; ++e) a[e] = kt[(4 * e + g) * kLd + 16 * nt + c];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < NW; ++mt)
           acc[mt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb[mt], acc[mt][j], 0, 0, 0);
       }
     }
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   __syncthreads();
   // lane (c, g) holds latent dims 16 nt + 4 g .. + 3 of row 16 mt + c
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
+  for (int mt = 0; mt < NW; ++mt) {
     const int r = 16 * mt + c;
     const int rt = r / hc, rh = r % hc;
     if (!(rt < ntok && rh < nh)) continue;
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const long trow = r0 + tok0 + rt;
 #pragma unroll
     for (int j = 0; j < NPW; ++j) {
-      const int d = 16 * (wave + 4 * j) + 4 * g;
+      const int d = 16 * (wave + NW * j) + 4 * g;
       if (d >= kv_rank) continue;  // kv_rank % 8 == 0: the four dims are inside together
       if (partial) {
         float* dst = ws_acc + (((long)blockIdx.z * heads + h0 + rh) * ws_rows + (trow - row_base)) * kv_rank + d;
@@ -312,26 +313,33 @@ __global__ __launch_bounds__(128) void latent_attention_reduce_kernel(
   }
 }
 
-template <int KS, int NPW>
-void launch_mfma(unsigned short* o_lat, const unsigned short* qc, const unsigned short* proj, long proj_ld,
+template <int KS, int NPW, int NW>
+bool launch_mfma(unsigned short* o_lat, const unsigned short* qc, const unsigned short* proj, long proj_ld,
                  const unsigned short* cache, int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
                  int bt_width, int seq0, int seq1, int rows_bound, int T, int heads, int rot_dim, int kv_rank,
                  int gate_off, float scale, int window, int nparts, int part_keys, float* ws_acc, float* ws_ml,
                  int row_base, hipStream_t s) {
-  constexpr int kLd = KtLd<KS>::v;
+  constexpr int kLd = KtLd<KS>::v, kRows = 16 * NW;
   constexpr size_t smem = kKeys * kLd * 2 + kRows * kKeys * 4 + kRows * kPLd * 2 + 3 * kRows * 4;
-  static_assert(smem <= 64 * 1024, "LDS");
+  static_assert(smem <= 160 * 1024, "LDS");
+  auto* fn = &latent_attention_mfma_kernel<KS, NPW, NW>;
+  if (smem > 64 * 1024) {  // once per kernel: more dynamic LDS than the default limit
+    static const bool ok = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess;
+    if (!ok) return false;
+  }
   const int hc = min(heads, kRows);
-  // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the 64 rows
+  // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the rows
   const int tq = nparts > 1 ? 1 : kRows / hc;
   dim3 grid(rows_bound / tq + (seq1 - seq0), (heads + hc - 1) / hc, nparts);
-  latent_attention_mfma_kernel<KS, NPW><<<grid, 256, smem, s>>>(
-      o_lat, qc, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, T, heads,
-      rot_dim, kv_rank, gate_off, scale, window, part_keys, ws_acc, ws_ml, row_base, rows_bound);
+  fn<<<grid, 64 * NW, smem, s>>>(o_lat, qc, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,
+                                tq, hc, T, heads, rot_dim, kv_rank, gate_off, scale, window, part_keys, ws_acc, ws_ml,
+                                row_base, rows_bound);
   if (nparts > 1)
     latent_attention_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(o_lat, ws_acc, ws_ml, proj, proj_ld, gate_off,
                                                                          nparts, heads, rows_bound, row_base, T,
                                                                          kv_rank);
+  return true;
 }
 
 }  // namespace
@@ -355,14 +363,16 @@ void launch_latent_attention_mfma(void* o_lat, const void* qc, const void* proj,
                                   float* ws_acc, float* ws_ml, int row_base, hipStream_t s) {
   if (seq1 <= seq0 || rows_bound <= 0) return;
   const int Dk = kv_rank + rot_dim;
-#define HS_LA(KS, NPW)                                                                                              \
-  launch_mfma<KS, NPW>((unsigned short*)o_lat, (const unsigned short*)qc, (const unsigned short*)proj, proj_ld,     \
-                       (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,      \
-                       rows_bound, T, heads, rot_dim, kv_rank, gate_off, scale, window, nparts, part_keys, ws_acc,   \
-                       ws_ml, row_base, s)
-  if (kv_rank <= 128 && Dk <= 192) HS_LA(6, 2);
-  else if (kv_rank <= 256 && Dk <= 320) HS_LA(10, 4);
-  else HS_LA(20, 8);
+#define HS_LA(KS, NPW, NW)                                                                                          \
+  launch_mfma<KS, NPW, NW>((unsigned short*)o_lat, (const unsigned short*)qc, (const unsigned short*)proj, proj_ld,  \
+                           (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,   \
+                           rows_bound, T, heads, rot_dim, kv_rank, gate_off, scale, window, nparts, part_keys, ws_acc, \
+                           ws_ml, row_base, s)
+  // (an 8-wave / 128-row variant, NW = 8, halves the tile fetches per row but was not faster: 1107 vs 1019 us
+  // at 8192 tokens x 16 heads, its 512-thread launch bound caps it at 128 registers and it spills)
+  if (kv_rank <= 128 && Dk <= 192) HS_LA(6, 2, 4);
+  else if (kv_rank <= 256 && Dk <= 320) HS_LA(10, 4, 4);
+  else HS_LA(20, 8, 4);
 #undef HS_LA
 }
 

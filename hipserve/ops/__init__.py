@@ -192,7 +192,7 @@ class KernelOps:
     LATENT_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x up to 4 heads = 16 waves)
     # bf16 runs the MFMA kernel (HIPSERVE_LATENT_MFMA=0: the generic kernel, as fp32 does)
     LATENT_MFMA = os.environ.get("HIPSERVE_LATENT_MFMA", "1") != "0"
-    LATENT_DECODE_RUN = 64   # keys per run of a decode row (a multiple of 32)
+    LATENT_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32; 64 measured slower)
 
     def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
                          gate_off, scale, window):
@@ -234,7 +234,26 @@ class KernelOps:
         self._seq.mingru_scan(y, state, proj, b_z, b_x, meta.seq_cu, meta.seq_ctx, meta.seq_state, meta.max_q)
 
     def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
-        self._seq.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
+        if E <= 128:
+            self._seq.moe_align(experts, E, tile, slots, tile_expert, pair_slot)
+            return
+        # more experts than the alignment kernel's LDS tables hold: the same layout from device-side
+        # sort / scan ops (no host round trip)
+        ex = experts.long()
+        P = ex.numel()
+        order = torch.argsort(ex, stable=True)
+        counts = torch.bincount(ex, minlength=E)
+        padded = (counts + tile - 1) // tile * tile
+        ends = torch.cumsum(padded, 0)
+        first = torch.cumsum(counts, 0) - counts           # rank of each expert's first pair in `order`
+        e_sorted = ex[order]
+        pos = (ends - padded)[e_sorted] + torch.arange(P, device=ex.device) - first[e_sorted]
+        slots.fill_(-1)
+        slots[pos] = order.to(torch.int32)
+        pair_slot[order] = pos.to(torch.int32)
+        t = torch.arange(tile_expert.numel(), device=ex.device) * tile
+        te = torch.searchsorted(ends, t, right=True)
+        tile_expert.copy_(torch.where(te < E, te, torch.full_like(te, -1)).to(torch.int32))
 
     def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
         self._seq.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)

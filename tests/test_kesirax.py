@@ -153,7 +153,7 @@ def test_mingru_alone(target, width):
 
 
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("top,experts,ff", [(1, 3, 12), (2, 4, 20), (3, 5, 70)])
+@pytest.mark.parametrize("top,experts,ff", [(1, 3, 12), (2, 4, 20), (3, 5, 70), (2, 130, 8)])
 def test_table_moe_and_residual_update_alone(target, top, experts, ff):
     dev, dt = torch.device(target[0]), getattr(torch, target[1])
     f = O.moe(experts=experts, top=top, ff=ff)
@@ -385,3 +385,35 @@ def test_graph_decode_matches_eager_gpu(tmp_path):
             assert row[t] >= row.max() - 0.15, (k, t, int(row.argmax()))
     same = sum(a == b for a, b in zip(outs[0], outs[1]))
     assert same >= len(prompts) - 1, (outs[0], outs[1])  # bf16 near-ties may flip one continuation
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kv_rank,window", [(64, 300), (136, 0)])
+def test_latent_attention_long_prompt_gpu(kv_rank, window):
+    """A prompt portion with tens of thousands of (token, head) rows on the matrix-core kernel: many key
+    tiles per row, two sequences of unequal length and interleaved pages in one step."""
+    dev, dt = torch.device("cuda"), torch.bfloat16
+    l = O.attn_layer(heads=16, dim=16, rot_dim=8, vdim=16, q_rank=24, kv_rank=kv_rank, window=window)
+    cfg = O.make_config([l], width=32)
+    W = O.make_weights(cfg, seed=31)
+    n = (1500, 700)
+    g = torch.Generator().manual_seed(7)
+    hs = [torch.randn(k, 32, generator=g).bfloat16().float() for k in n]
+    want = torch.cat([O.latent_attention(h, W, "l0.mix.", l["mixer"], 1e-6) for h in hs])
+    mix = LatentAttention(HybridConfig.from_dict(cfg).layers[0].mixer, 32, 1e-6, dev, dt, get_ops(dev))
+    mix.load(lambda k: W[k], "l0.mix.")
+    bs, T = 16, sum(n)
+    nb = [-(-k // bs) for k in n]
+    bt = torch.zeros(2, max(nb), dtype=torch.int32)
+    bt[0, :nb[0]] = torch.arange(nb[0], dtype=torch.int32) * 2 + 1     # interleaved pages
+    bt[1, :nb[1]] = torch.arange(nb[1], dtype=torch.int32) * 2
+    pos = torch.cat([torch.arange(k) for k in n])
+    seq = torch.cat([torch.full((k,), i) for i, k in enumerate(n)])
+    slots = bt.long()[seq, pos // bs] * bs + pos % bs
+    meta = AttnMeta(num_prefill_tokens=T, num_decode=0, positions=pos.to(dev), slot_mapping=slots.to(dev),
+                    seq_cu=torch.tensor([0, n[0], T], dtype=torch.int32, device=dev),
+                    seq_ctx=torch.tensor(n, dtype=torch.int32, device=dev), seq_bt=bt.to(dev), max_q=max(n),
+                    max_ctx=max(n))
+    cache = torch.zeros(mix.cache_shape(2 * max(nb) + 2, bs), device=dev, dtype=dt)
+    got = mix.forward(torch.cat(hs).to(dev, dt), meta, cache)
+    assert rel_err(got, want) < TOL["bfloat16"]
