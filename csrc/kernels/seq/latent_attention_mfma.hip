@@ -6,13 +6,13 @@
 // latent_attention_mfma: a workgroup (4 waves) owns 64 (token, head) rows of one sequence, tokens
 // consecutive, so all rows share one run of keys. Per 32-key tile:
 //   1. the tile's cache rows [32][Dk] go to LDS row-major; wave w computes S = K . Q^T for its 16 rows
-//      (mfma_f32_16x16x32_bf16, the Q operands stay in registers) and writes it to LDS as fp32;
-//   2. four threads per row do the masked online softmax in fp32 (max, exp, sum, rescale factor) and
-//      write P as bf16;
+//      (mfma_f32_16x16x32_bf16, the Q operands stay in registers);
+//   2. the same wave does the masked online softmax in fp32 on the scores in its registers (a row's 32
+//      scores sit in four lanes) and writes P as bf16 to LDS for all waves;
 //   3. every wave owns a slice of the latent dims for ALL 64 rows: acc = acc * alpha + V^T . P^T. The
 //      contraction index is the key, so the V operand is read column-wise from the same row-major K
-//      tile (eight 2-byte LDS reads per operand; the MFMA's k slots are dealt to keys 4 e + g so that
-//      the four rows read together hit disjoint banks, and P is stored in that key order).
+//      tile (eight 2-byte LDS reads per operand); the MFMA's k slots are dealt to the keys in the order the
+//      score registers hold them, so P needs no shuffle.
 // Decode rows (one token, many keys) split their keys over grid.z; latent_attention_reduce merges the
 // runs' (max, sum, output).
 // The output (latent space, times the head's sigmoid gate, over the softmax sum) is written as bf16.
@@ -69,15 +69,15 @@ HS_DEVICE bool find_tile64(const int* __restrict__ seq_cu, int seq0, int seq1, i
   return false;
 }
 
-// K tile row stride: 32 KS + pad with stride / 2 = 8 (mod 32) dwords, so that the four key rows a wave
-// reads together in the P . V operand loads fall into disjoint LDS banks; a multiple of 8 elements.
-template <int KS> struct KtLd { static constexpr int v = KS * 32 + ((KS & 1) ? 48 : 16); };
+// K tile row stride: 32 KS + 8 elements (16-byte aligned rows; stride / 2 = 4 (mod 16) dwords keeps both the
+// row-wise 16-byte operand reads of S and the column-wise 2-byte reads of P . V at two-way bank conflicts).
+template <int KS> struct KtLd { static constexpr int v = KS * 32 + 8; };
 
 // KS: 32-dim steps of a cache row (Dk <= 32 KS); NPW: 16-dim output tiles per wave (kv_rank <= 64 NPW).
 // grid.z > 1 splits the keys of a row into runs of part_keys; the runs' unnormalised outputs and
 // (max, sum) go to ws_acc / ws_ml for latent_attention_reduce (decode rows: many keys, few rows).
 template <int KS, int NPW, int NW>
-__global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
+__global__ __launch_bounds__(64 * NW, 2) void latent_attention_mfma_kernel(
     unsigned short* __restrict__ o_lat, const unsigned short* __restrict__ qc, const unsigned short* __restrict__ proj,
     long proj_ld, const unsigned short* __restrict__ cache, int block_size, const int* __restrict__ seq_cu,
     const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
@@ -87,11 +87,10 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
   constexpr int kRows = 16 * NW, kThreads = 64 * NW, kFT = kThreads / kKeys;  // kFT threads fill one key's row
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned short* kt = reinterpret_cast<unsigned short*>(smem);                    // [32][kLd] bf16 cache rows
-  float* s_lds = reinterpret_cast<float*>(smem + kKeys * kLd * 2);                 // [64][32] fp32 scores
-  unsigned short* p_lds = reinterpret_cast<unsigned short*>(s_lds + kRows * kKeys);  // [64][kPLd] bf16, keys permuted
-  float* alpha = reinterpret_cast<float*>(p_lds + kRows * kPLd);                   // [64]
-  float* m_run = alpha + kRows;                                                    // [64]
-  float* l_run = m_run + kRows;                                                    // [64]
+  unsigned short* p_lds = kt + kKeys * kLd;                                        // [rows][kPLd] bf16, MFMA k order
+  float* alpha = reinterpret_cast<float*>(p_lds + kRows * kPLd);                   // [rows]
+  float* m_lds = alpha + kRows;                                                    // [rows] (epilogue)
+  float* l_lds = m_lds + kRows;                                                    // [rows] (epilogue)
   int s, tok0;
   // (workgroups are dealt to the XCDs round-robin; giving each XCD a contiguous run of token tiles was
   // measured slower, 1188 vs 1013 us at 8192 tokens x 16 heads: the causal start makes the runs unequal)
@@ -121,7 +120,6 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
       qf[ks] = __builtin_bit_cast(bf16x8, v);
     }
   }
-  if (tid < kRows) { m_run[tid] = -INFINITY; l_run[tid] = 0.f; }
   f32x4 acc[NW][NPW];
 #pragma unroll
   for (int mt = 0; mt < NW; ++mt)
@@ -131,12 +129,14 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
   const int chunks = Dk / 8;  // 16-byte chunks of a cache row
   // tile fill: kFT threads per key, each its key's chunks fk, fk + kFT, ...
   const int fkey = tid / kFT, fk = tid % kFT;
-  // softmax: 4 threads per row; thread `part` owns the keys 4 e + part (e = 0..7) of the tile
-  const int sr = tid >> 2, part = tid & 3;
+  // softmax: the wave that computed a row's scores keeps them; lane (c, g) owns row 16 wave + c and the keys
+  // 16 nt + 4 g + i of a tile (nt = 0, 1; i = 0..3) = the MFMA k slot (g, e = 4 nt + i) of P . V below
+  const int sr = 16 * wave + c;
   const int srt = sr / hc, srh = sr % hc;
   const bool sact = srt < ntok && srh < nh;
   const int spos = p_first + srt;
   const int s_lo = window > 0 ? max(0, spos - window + 1) : 0;
+  float m_run = -INFINITY, l_run = 0.f;
   constexpr int kFill = (KS * 4 + kFT - 1) / kFT;
   u16x8 fv[kFill];
   // the thread's part of a tile, all loads in flight together; zero past Dk and past the last key
@@ -151,15 +151,14 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
       if (in && ch < chunks) fv[i] = *reinterpret_cast<const u16x8*>(cache + kr + 8 * ch);
     }
   };
-  if (lo <= hi) fetch(lo);
   for (int j0 = lo; j0 <= hi; j0 += kKeys) {
+    fetch(j0);        // (prefetching a tile ahead costs 40 registers and the second workgroup per CU)
     __syncthreads();  // the previous tile's reads of the K tile (P . V) are done
 #pragma unroll
     for (int i = 0; i < kFill; ++i) {
       const int ch = fk + kFT * i;
       if (ch < KS * 4) *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = fv[i];
     }
-    if (j0 + kKeys <= hi) fetch(j0 + kKeys);  // the next tile travels while this one is computed
     __syncthreads();
     // 1. S^T tiles: a = keys (16 per tile), b = this wave's 16 query rows
     f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -171,27 +170,21 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
         sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[ks], sc[nt], 0, 0, 0);
       }
     }
-    // lane (c, g) holds keys 16 nt + 4 g .. + 3 of row 16 wave + c
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-      *reinterpret_cast<f32x4*>(s_lds + (16 * wave + c) * kKeys + 16 * nt + 4 * g) = sc[nt];
-    __syncthreads();
-    // 2. online softmax in fp32; P as bf16 with key kk at position 8 (kk % 4) + kk / 4 (the MFMA's k order below)
+    // 2. online softmax in fp32 on the scores in registers (lane (c, g): keys 16 nt + 4 g + i of row sr; the
+    //    row's four lanes meet through two shuffles); P as bf16 in the k order of the MFMA below
     {
       float v[8];
       float mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int kk = 4 * e + part;
-        const int j = j0 + kk;
+        const int j = j0 + 16 * (e >> 2) + 4 * g + (e & 3);
         const bool vis = sact && j <= hi && j <= spos && j >= s_lo;
-        v[e] = vis ? s_lds[sr * kKeys + kk] * scale : -INFINITY;
+        v[e] = vis ? sc[e >> 2][e & 3] * scale : -INFINITY;
         mx = fmaxf(mx, v[e]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-      const float mo = m_run[sr];
-      const float mn = fmaxf(mo, mx);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m_run, mx);
       float sum = 0.f;
       u16x8 pk;
 #pragma unroll
@@ -201,19 +194,17 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
         pk[e] = pb;
         sum += bf16_to_f32(pb);  // the sum of the weights that are actually multiplied
       }
-      sum += __shfl_xor(sum, 1, 64);
-      sum += __shfl_xor(sum, 2, 64);
-      *reinterpret_cast<u16x8*>(p_lds + sr * kPLd + 8 * part) = pk;
-      if (part == 0) {
-        const float al = (mn > -INFINITY) ? expf(mo - mn) : 1.f;  // mo = -inf: 0
-        alpha[sr] = al;
-        l_run[sr] = l_run[sr] * al + sum;
-        m_run[sr] = mn;
-      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      *reinterpret_cast<u16x8*>(p_lds + sr * kPLd + 8 * g) = pk;
+      const float al = (mn > -INFINITY) ? __expf(m_run - mn) : 1.f;  // m_run = -inf: 0
+      if (g == 0) alpha[sr] = al;
+      l_run = l_run * al + sum;
+      m_run = mn;
     }
     __syncthreads();
     // 3. acc[rows][dims] = acc * alpha + V^T . P^T: a = 16 latent dims, b = 16 rows; the MFMA's k slot
-    //    (g, e) is key 4 e + g, read column-wise from the row-major K tile
+    //    (g, e) is key 16 (e / 4) + 4 g + e % 4, read column-wise from the row-major K tile
     bf16x8 pb[NW];
     float al[NW];
     bool rescale = false;
@@ -235,13 +226,14 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
       if (nt < ntiles_dv) {
         u16x8 a;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) a[e] = kt[(4 * e + g) * kLd + 16 * nt + c];
+        for (int e = 0; e < 8; ++e) a[e] = kt[(16 * (e >> 2) + 4 * g + (e & 3)) * kLd + 16 * nt + c];
 #pragma unroll
         for (int mt = 0; mt < NW; ++mt)
           acc[mt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb[mt], acc[mt][j], 0, 0, 0);
       }
     }
   }
+  if (g == 0) { m_lds[sr] = m_run; l_lds[sr] = l_run; }
   __syncthreads();
   const bool partial = gridDim.z > 1;
   if (tid < kRows) {  // alpha <- gate / softmax sum of the row (1 for partial results)
@@ -251,11 +243,11 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_mfma_kernel(
     if (act && partial) {
       f = 1.f;
       const long wrow = (long)blockIdx.z * heads * ws_rows + (long)(h0 + rh) * ws_rows + (r0 + tok0 + rt - row_base);
-      ws_ml[2 * wrow] = m_run[tid];
-      ws_ml[2 * wrow + 1] = l_run[tid];
-    } else if (act && l_run[tid] > 0.f) {
+      ws_ml[2 * wrow] = m_lds[tid];
+      ws_ml[2 * wrow + 1] = l_lds[tid];
+    } else if (act && l_lds[tid] > 0.f) {
       const float gt = bf16_to_f32(proj[(long)(r0 + tok0 + rt) * proj_ld + gate_off + h0 + rh]);
-      f = sigmoid_f(gt) / l_run[tid];
+      f = sigmoid_f(gt) / l_lds[tid];
     }
     alpha[tid] = f;
   }
@@ -320,7 +312,7 @@ bool launch_mfma(unsigned short* o_lat, const unsigned short* qc, const unsigned
                  int gate_off, float scale, int window, int nparts, int part_keys, float* ws_acc, float* ws_ml,
                  int row_base, hipStream_t s) {
   constexpr int kLd = KtLd<KS>::v, kRows = 16 * NW;
-  constexpr size_t smem = kKeys * kLd * 2 + kRows * kKeys * 4 + kRows * kPLd * 2 + 3 * kRows * 4;
+  constexpr size_t smem = kKeys * kLd * 2 + kRows * kPLd * 2 + 3 * kRows * 4;
   static_assert(smem <= 160 * 1024, "LDS");
   auto* fn = &latent_attention_mfma_kernel<KS, NPW, NW>;
   if (smem > 64 * 1024) {  // once per kernel: more dynamic LDS than the default limit
