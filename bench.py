@@ -286,7 +286,7 @@ def orchestrate(args) -> int:
 
 def main():
     args = parse()
-    if args.layer_compare:  # its own single-GPU workload; the headline contract below is untouched
+    if args.layer_compare:  # its own single-GPU workload; the headline benchmark below is untouched
         from hipserve.bench.layer_compare import main as layer_compare
 
         sys.exit(layer_compare(args))

@@ -12,11 +12,12 @@ Input, one JSON object per line on stdin::
 
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": ["a"]}
 
-``entries``: each request's next tokens and the offsets among them whose logits are
-wanted; ``end``: requests that are finished after the step (their cache blocks and
-state slot are given back). A step with wanted rows writes ``<out>/<step>.f32``
-(little-endian float32 [rows, vocab], in entry and ``want`` order); every step answers
-``done <step>`` on stdout.
+``entries`` lists, per request id, the tokens to append now and ``want``, offsets into
+those tokens whose logits should be written; a request id seen for the first time starts
+a new sequence. ``end`` names requests to drop once the step has run: their cache blocks
+and their state slot return to the pools. If any row is wanted the step writes
+``<out>/<step>.f32`` (little-endian float32 [rows, vocab], rows ordered by entry, then by
+``want``); after every step a line ``done <step>`` goes to stdout.
 """
 from __future__ import annotations
 

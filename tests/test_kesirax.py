@@ -417,3 +417,70 @@ def test_latent_attention_long_prompt_gpu(kv_rank, window):
     cache = torch.zeros(mix.cache_shape(2 * max(nb) + 2, bs), device=dev, dtype=dt)
     got = mix.forward(torch.cat(hs).to(dev, dt), meta, cache)
     assert rel_err(got, want) < TOL["bfloat16"]
+
+
+def test_openai_server_and_cli_config(tmp_path):
+    """The engine command line resolves a checkpoint folder of this design (model class by config.json) and
+    the OpenAI server completes, streams and samples with penalties and logprobs on it."""
+    import asyncio
+
+    import aiohttp
+    from aiohttp import web
+
+    from hipserve.server.api_server import OpenAIServer
+    from hipserve.server.async_engine import AsyncEngine
+    from hipserve.server.cli import build_parser, config_from_args
+
+    cfg = base_config()
+    path = O.save_checkpoint(str(tmp_path / "srv"), cfg, O.make_weights(cfg, seed=41))
+    a = build_parser().parse_args(["--model", path, "--served-model-name", "kx", "--device", "cpu", "--dtype", "float32",
+                                   "--max-model-len", "256", "--max-num-seqs", "4", "--num-kv-blocks", "64",
+                                   "--max-num-batched-tokens", "32"])
+    ecfg = config_from_args(a)
+
+    async def main():
+        eng = LLMEngine(ecfg, tp=TPGroup())
+        assert type(eng.runner.model).__name__ == "KesiraxModel" and eng.states is not None
+        ae = AsyncEngine(eng)
+        ae.start(asyncio.get_running_loop())
+        runner = web.AppRunner(OpenAIServer(ae, "kx", eng.max_model_len).app())
+        await runner.setup()
+        site = web.TCPSite(runner, "127.0.0.1", 0)
+        await site.start()
+        port = site._server.sockets[0].getsockname()[1]
+        try:
+            async with aiohttp.ClientSession() as s:
+                body = {"model": "kx", "prompt": [5, 9, 33, 70, 2, 41] * 9, "max_tokens": 6, "temperature": 0.7,
+                        "top_p": 0.9, "seed": 3, "presence_penalty": 0.5, "logprobs": 2}
+                async with s.post(f"http://127.0.0.1:{port}/v1/completions", json=body) as r:
+                    assert r.status == 200
+                    d = await r.json()
+                    assert d["usage"]["completion_tokens"] == 6 and d["usage"]["prompt_tokens"] == 54
+                async with s.post(f"http://127.0.0.1:{port}/v1/completions", json=body) as r:
+                    assert (await r.json())["choices"][0]["text"] == d["choices"][0]["text"]   # seeded: repeatable
+        finally:
+            await runner.cleanup()
+            ae.stop() if hasattr(ae, "stop") else None
+
+    asyncio.run(main())
+
+
+def test_preemption_recomputes_state(tmp_path):
+    """A cache pool too small for all running requests: the scheduler preempts (blocks and state slot freed,
+    recomputed later from position 0 in whichever slot is free) and the outputs stay the oracle's argmaxes."""
+    cfg = base_config()
+    W = O.make_weights(cfg, seed=43)
+    path = O.save_checkpoint(str(tmp_path / "pre"), cfg, W)
+    ecfg = EngineConfig(model=path, dtype="float32", device="cpu", max_num_seqs=4, max_num_batched_tokens=32,
+                        num_kv_blocks=13, max_model_len=128, enforce_eager=True)
+    eng = LLMEngine(ecfg, tp=TPGroup())
+    prompts = [tokens(n, cfg["vocab"], 60 + n) for n in (40, 33, 45, 38)]
+    res = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True))
+    assert eng.scheduler.num_preemptions > 0
+    for p, (out, _text, reason) in zip(prompts, res):
+        assert len(out) == 24 and reason == "length"
+        lg = O.forward(cfg, W, p + out)
+        for k, t in enumerate(out):
+            row = lg[len(p) + k - 1]
+            assert row[t] >= row.max() - 1e-3, (k, t, int(row.argmax()))
+    assert eng.states.num_free() == 4 and eng.blocks.num_free() == eng.blocks.num_blocks
