@@ -484,3 +484,68 @@ def test_preemption_recomputes_state(tmp_path):
             row = lg[len(p) + k - 1]
             assert row[t] >= row.max() - 1e-3, (k, t, int(row.argmax()))
     assert eng.states.num_free() == 4 and eng.blocks.num_free() == eng.blocks.num_blocks
+
+
+def random_config(seed):
+    """A random small model: sizes, layer order, loop, windows and constants drawn per seed."""
+    import random
+
+    r = random.Random(seed)
+    groups = r.choice([1, 2, 3, 4])
+    width = groups * r.choice([8, 12, 20])
+    vocab = r.choice([37, 64, 101])
+
+    def mlp():
+        if r.random() < 0.2:
+            return None
+        e = r.choice([1, 2, 3, 5, 6])
+        return O.moe(experts=e, top=r.randint(1, min(e, 3)), ff=r.choice([4, 10, 24, 33]))
+
+    layers = []
+    for _ in range(r.randint(2, 5)):
+        if r.random() < 0.5:
+            layers.append(O.gru_layer(width=r.choice([8, 36, 70, 130]), mlp=mlp()))
+        else:
+            rot = r.choice([2, 4, 8, 16])
+            layers.append(O.attn_layer(heads=r.randint(1, 9), dim=r.choice([4, 8, 16, 24]), rot_dim=rot,
+                                       rot_dims=r.choice([rot, rot, max(2, rot // 2)]), vdim=r.choice([4, 8, 20]),
+                                       q_rank=r.choice([6, 16, 28]), kv_rank=r.choice([8, 24, 40, 72]),
+                                       window=r.choice([0, 2, 5, 17, 64]), base=r.choice([10.0, 1e4, 5e5]),
+                                       scale=r.choice([None, 0.3, 0.05]), mlp=mlp()))
+    a = r.randint(0, len(layers) - 1)
+    b = r.randint(a, len(layers))
+    return O.make_config(layers, width=width, vocab=vocab, loop=(a, b, r.randint(1, 3)), groups=groups,
+                         logit_scale=r.choice([0.25, 1.0, 3.0]), eps=r.choice([1e-6, 1e-5]))
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("seed", range(8))
+def test_random_models(tmp_path, target, seed):
+    """Random sizes and layer orders: whole prompts, random portions with decoded tails, and two requests
+    interleaved in one batch, against whole-sequence oracle logits."""
+    import random
+
+    cfg = random_config(seed)
+    W = O.make_weights(cfg, seed=100 + seed)
+    r = random.Random(1000 + seed)
+    ta, tb = tokens(r.randint(30, 60), cfg["vocab"], 200 + seed), tokens(r.randint(3, 40), cfg["vocab"], 300 + seed)
+    ra, rb = O.forward(cfg, W, ta), O.forward(cfg, W, tb)
+    sess = session(tmp_path, cfg, W, target, max_tokens=256)
+    check_all(replay(sess, portions(ta, [len(ta)])), "a", ra, TOL[target[1]])
+    check_all(replay(sess, portions(ta, [r.randint(2, 9) for _ in range(5)])), "a", ra, TOL[target[1]])
+    steps, pa, pb = [], 0, 0
+    while pa < len(ta) or pb < len(tb):
+        step = []
+        for rid, t, p in (("a", ta, pa), ("b", tb, pb)):
+            if p < len(t) and r.random() < 0.8:
+                n = min(r.choice([1, 1, 2, 3, 7]), len(t) - p)
+                step.append((rid, t[p:p + n], list(range(n)), p + n == len(t)))
+                if rid == "a":
+                    pa += n
+                else:
+                    pb += n
+        if step:
+            steps.append(step)
+    got = replay(sess, steps)
+    check_all(got, "a", ra, TOL[target[1]])
+    check_all(got, "b", rb, TOL[target[1]])
