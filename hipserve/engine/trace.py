@@ -105,7 +105,7 @@ def build_engine(model: str, dtype: str, max_tokens: int, device: str | None = N
     from .llm_engine import LLMEngine
 
     device = device or ("cuda" if torch.cuda.is_available() else "cpu")
-    blocks = -(-max_tokens // block_size) + MAX_LIVE + 1   # + the runner's scratch block
+    blocks = -(-max_tokens // block_size) + 1   # the pool holds max_tokens; + the runner's scratch block
     cfg = EngineConfig(model=model, load_format="safetensors", dtype=dtype, device=device, block_size=block_size,
                        max_num_seqs=MAX_LIVE, max_num_batched_tokens=max(max_tokens, 64), num_kv_blocks=blocks,
                        max_model_len=max(max_tokens, 64), enable_prefix_caching=False, enforce_eager=True)
