@@ -32,7 +32,8 @@ __global__ __launch_bounds__(256) void latent_q_cat_kernel(unsigned short* __res
   const int Dk = kv_rank + rot_dim;
   unsigned short* dst = qc + ((long)h * T + t) * Dk;
   const float* qa = q_abs + ((long)h * T + t) * kv_rank;
-  for (int e = threadIdx.x; e < kv_rank; e += 256) dst[e] = f32_to_bf16(qa[e]);
+  if (q_abs != nullptr)  // else the absorbed part is already in qc (written by the absorption GEMM)
+    for (int e = threadIdx.x; e < kv_rank; e += 256) dst[e] = f32_to_bf16(qa[e]);
   const unsigned short* qr = q + (long)t * heads * (dim + rot_dim) + (long)h * (dim + rot_dim) + dim;
   const float pos = (float)positions[t];
   for (int e = threadIdx.x; e < rot_dim; e += 256) {
@@ -278,30 +279,29 @@ __global__ __launch_bounds__(64 * NW, 2) void latent_attention_mfma_kernel(
 }
 
 // o_lat[h, row_base + r, :] = sum_p acc_p e^(m_p - M) / sum_p l_p e^(m_p - M) * sigmoid(gate)
+constexpr int kMaxRuns = 64;
 __global__ __launch_bounds__(128) void latent_attention_reduce_kernel(
     unsigned short* __restrict__ o_lat, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
     const unsigned short* __restrict__ proj, long proj_ld, int gate_off, int nparts, int heads, int ws_rows,
     int row_base, int T_rows, int kv_rank) {
-  const int r = blockIdx.x, h = blockIdx.y;
-  float M = -INFINITY;
-  for (int p = 0; p < nparts; ++p) M = fmaxf(M, ws_ml[2 * (((long)p * heads + h) * ws_rows + r)]);
-  float L = 0.f;
-  for (int p = 0; p < nparts; ++p) {
-    const long w = ((long)p * heads + h) * ws_rows + r;
-    const float m = ws_ml[2 * w];
-    if (m > -INFINITY) L += ws_ml[2 * w + 1] * expf(m - M);
+  __shared__ float sc[kMaxRuns];  // each run's weight e^(m_p - M) / L * gate, 0 for empty runs
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  if (tid < 64) {  // one wave: run p on lane p
+    const long w = ((long)min(tid, nparts - 1) * heads + h) * ws_rows + r;
+    const float m = tid < nparts ? ws_ml[2 * w] : -INFINITY;
+    const float l = tid < nparts ? ws_ml[2 * w + 1] : 0.f;
+    const float M = wave_max(m);
+    const float e = m > -INFINITY ? __expf(m - M) : 0.f;
+    const float L = wave_sum(l * e);
+    const float gate = sigmoid_f(bf16_to_f32(proj[(long)(row_base + r) * proj_ld + gate_off + h]));
+    sc[tid] = L > 0.f ? e * gate / L : 0.f;
   }
+  __syncthreads();
   const long trow = row_base + r;
-  const float gate = sigmoid_f(bf16_to_f32(proj[trow * proj_ld + gate_off + h]));
-  const float f = L > 0.f ? gate / L : 0.f;
-  for (int d = threadIdx.x; d < kv_rank; d += 128) {
+  for (int d = tid; d < kv_rank; d += 128) {
     float o = 0.f;
-    for (int p = 0; p < nparts; ++p) {
-      const long w = ((long)p * heads + h) * ws_rows + r;
-      const float m = ws_ml[2 * w];
-      if (m > -INFINITY) o += ws_acc[w * kv_rank + d] * expf(m - M);
-    }
-    o_lat[((long)h * T_rows + trow) * kv_rank + d] = f32_to_bf16(o * f);
+    for (int p = 0; p < nparts; ++p) o += ws_acc[(((long)p * heads + h) * ws_rows + r) * kv_rank + d] * sc[p];
+    o_lat[((long)h * T_rows + trow) * kv_rank + d] = f32_to_bf16(o);
   }
 }
 

@@ -102,22 +102,23 @@ void latent_attention(at::Tensor& o_lat, const at::Tensor& q_abs, const at::Tens
 }
 
 // bf16 prompt portions on the matrix cores: qc (scratch) [heads, T, kv_rank + rot_dim] is filled here.
-void latent_attention_mfma(at::Tensor& o_lat, at::Tensor& qc, const at::Tensor& q_abs, const at::Tensor& q,
+void latent_attention_mfma(at::Tensor& o_lat, at::Tensor& qc, const c10::optional<at::Tensor>& q_abs, const at::Tensor& q,
                            const at::Tensor& proj, const at::Tensor& positions, const at::Tensor& cache,
                            const at::Tensor& seq_cu, const at::Tensor& seq_ctx, const at::Tensor& seq_bt, int64_t seq0,
                            int64_t seq1, int64_t rows_bound, const at::Tensor& inv_freq, int64_t heads, int64_t dim,
                            int64_t rot_dim, int64_t kv_rank, int64_t gate_off, double scale, int64_t window,
                            int64_t nparts, int64_t part_keys, const c10::optional<at::Tensor>& ws_acc,
                            const c10::optional<at::Tensor>& ws_ml, int64_t row_base, bool fill_qc) {
-  CHECK_DEV(q); CHECK_CONTIG(o_lat); CHECK_CONTIG(qc); CHECK_F32(q_abs); CHECK_CONTIG(q); CHECK_CONTIG(cache);
+  CHECK_DEV(q); CHECK_CONTIG(o_lat); CHECK_CONTIG(qc); CHECK_CONTIG(q); CHECK_CONTIG(cache);
   CHECK_F32(inv_freq); CHECK_I32(seq_cu); CHECK_I32(seq_ctx); CHECK_I32(seq_bt);
+  if (q_abs.has_value()) CHECK_F32(*q_abs);
   TORCH_CHECK(q.scalar_type() == at::kBFloat16 && o_lat.scalar_type() == at::kBFloat16 &&
               qc.scalar_type() == at::kBFloat16 && cache.scalar_type() == at::kBFloat16 &&
               proj.scalar_type() == at::kBFloat16, "latent_attention_mfma: bf16 only");
   TORCH_CHECK(hipserve::latent_attention_mfma_ok(kv_rank, rot_dim), "latent_attention_mfma: unsupported latent sizes");
   const long T = q.size(0);
   TORCH_CHECK(q.dim() == 2 && q.size(1) == heads * (dim + rot_dim));
-  TORCH_CHECK(q_abs.numel() == heads * T * kv_rank && o_lat.numel() == heads * T * kv_rank &&
+  TORCH_CHECK((!q_abs.has_value() || q_abs->numel() == heads * T * kv_rank) && o_lat.numel() == heads * T * kv_rank &&
               qc.numel() == heads * T * (kv_rank + rot_dim));
   TORCH_CHECK(cache.dim() == 3 && cache.size(2) == kv_rank + rot_dim);
   TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T && proj.size(1) >= gate_off + heads);
@@ -126,7 +127,7 @@ void latent_attention_mfma(at::Tensor& o_lat, at::Tensor& qc, const at::Tensor& 
   TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_bt.dim() == 2 && seq_bt.size(0) >= nseq);
   TORCH_CHECK(0 <= seq0 && seq0 <= seq1 && seq1 <= nseq && rows_bound <= T && 2 * inv_freq.numel() <= rot_dim);
   float *wa = nullptr, *wm = nullptr;
-  TORCH_CHECK(nparts >= 1 && row_base >= 0 && row_base + rows_bound <= T);
+  TORCH_CHECK(nparts >= 1 && nparts <= 64 && row_base >= 0 && row_base + rows_bound <= T);
   if (nparts > 1) {
     TORCH_CHECK(part_keys > 0 && part_keys % 32 == 0 && ws_acc.has_value() && ws_ml.has_value());
     TORCH_CHECK(ws_acc->scalar_type() == at::kFloat && ws_acc->is_contiguous() &&
@@ -138,7 +139,8 @@ void latent_attention_mfma(at::Tensor& o_lat, at::Tensor& qc, const at::Tensor& 
   }
   c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
   if (fill_qc)
-    hipserve::launch_latent_q_cat(qc.data_ptr(), q_abs.data_ptr<float>(), q.data_ptr(), positions.data_ptr<long>(),
+    hipserve::launch_latent_q_cat(qc.data_ptr(), q_abs.has_value() ? q_abs->data_ptr<float>() : nullptr, q.data_ptr(),
+                                  positions.data_ptr<long>(),
                                   inv_freq.data_ptr<float>(), inv_freq.numel(), T, heads, dim, rot_dim, kv_rank,
                                   cur_stream());
   hipserve::launch_latent_attention_mfma(o_lat.data_ptr(), qc.data_ptr(), proj.data_ptr(), proj.stride(0),
@@ -212,7 +214,7 @@ TORCH_LIBRARY(hipserve_seq, m) {
   m.def("latent_attention(Tensor(a!) o_lat, Tensor q_abs, Tensor q, Tensor proj, Tensor cache, Tensor seq_cu, "
         "Tensor seq_ctx, Tensor seq_bt, int seq0, int seq1, int rows_bound, int tq, Tensor inv_freq, int heads, "
         "int dim, int rot_dim, int kv_rank, int gate_off, float scale, int window) -> ()");
-  m.def("latent_attention_mfma(Tensor(a!) o_lat, Tensor(b!) qc, Tensor q_abs, Tensor q, Tensor proj, Tensor positions, "
+  m.def("latent_attention_mfma(Tensor(a!) o_lat, Tensor(b!) qc, Tensor? q_abs, Tensor q, Tensor proj, Tensor positions, "
         "Tensor cache, Tensor seq_cu, Tensor seq_ctx, Tensor seq_bt, int seq0, int seq1, int rows_bound, "
         "Tensor inv_freq, int heads, int dim, int rot_dim, int kv_rank, int gate_off, float scale, int window, "
         "int nparts, int part_keys, Tensor(c!)? ws_acc, Tensor(d!)? ws_ml, int row_base, bool fill_qc) -> ()");

@@ -53,6 +53,7 @@ class LatentAttention:
         self.kv_norm = None    # [kv_rank] fp32
         self.w_uq = None       # [heads * (dim + rot_dim), q_rank]
         self.w_uk = None       # [heads, dim, kv_rank]
+        self.w_uk_wide = None  # [heads, dim, kv_rank + rot_dim], zero rotary columns (made at first use)
         self.w_uv_t = None     # [heads, kv_rank, vdim]
         self.w_o = None        # [hidden, heads * vdim]
         rd = s.rot_dims or s.rot_dim
@@ -96,7 +97,14 @@ class LatentAttention:
                            self.inv_freq, s.q_rank, s.kv_rank, s.rot_dim, self.eps)
         q = F.linear(cq, self.w_uq)                                    # [T, heads * (dim + rot_dim)]
         qh = q.view(T, s.heads, s.dim + s.rot_dim)
-        q_abs = _mm32(qh[:, :, : s.dim].transpose(0, 1), self.w_uk)    # [heads, T, kv_rank] fp32
+        if ops.latent_query_in_place(h.dtype, s.kv_rank, s.rot_dim):
+            # the absorption GEMM writes the attention kernel's query rows directly: bf16, the cached width,
+            # zero weight columns where the attention op puts the rotated part
+            if self.w_uk_wide is None:
+                self.w_uk_wide = F.pad(self.w_uk, (0, s.rot_dim)).contiguous()
+            q_abs = torch.bmm(qh[:, :, : s.dim].transpose(0, 1), self.w_uk_wide)   # [heads, T, kv_rank + rot_dim]
+        else:
+            q_abs = _mm32(qh[:, :, : s.dim].transpose(0, 1), self.w_uk)            # [heads, T, kv_rank] fp32
         o_lat = torch.empty(s.heads, T, s.kv_rank, device=h.device, dtype=h.dtype)
         ops.latent_attention(o_lat, q_abs, q, proj, cache, meta, self.inv_freq, s.heads, s.dim, s.rot_dim,
                              s.kv_rank, s.q_rank + s.key_dim, s.scale, s.window)

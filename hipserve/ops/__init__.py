@@ -194,6 +194,11 @@ class KernelOps:
     LATENT_MFMA = os.environ.get("HIPSERVE_LATENT_MFMA", "1") != "0"
     LATENT_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32; 64 measured slower)
 
+    def latent_query_in_place(self, dtype, kv_rank, rot_dim) -> bool:
+        """True when ``latent_attention`` wants the absorbed queries as bf16 rows of the cached width
+        ([heads, T, kv_rank + rot_dim], the rotary part left for it to fill) instead of fp32 [heads, T, kv_rank]."""
+        return dtype == torch.bfloat16 and self.LATENT_MFMA and bool(self._seq.latent_attention_mfma_ok(kv_rank, rot_dim))
+
     def latent_attention(self, o_lat, q_abs, q, proj, cache, meta, inv_freq, heads, dim, rot_dim, kv_rank,
                          gate_off, scale, window):
         """Prompt portions (the step's first sequences) run several tokens per workgroup, decode
@@ -203,7 +208,10 @@ class KernelOps:
         npf, Tp = nseq - nd, meta.num_prefill_tokens
         if (q.dtype == torch.bfloat16 and self.LATENT_MFMA and self._seq.latent_attention_mfma_ok(kv_rank, rot_dim)):
             # bf16: the matrix-core kernel; decode rows split their keys into runs merged by a reduce kernel
-            qc = torch.empty(heads, q.shape[0], kv_rank + rot_dim, device=q.device, dtype=q.dtype)
+            if q_abs.dtype == torch.bfloat16:  # the absorption GEMM wrote the rows in place (latent_query_in_place)
+                qc, q_abs = q_abs, None
+            else:
+                qc = torch.empty(heads, q.shape[0], kv_rank + rot_dim, device=q.device, dtype=q.dtype)
             fill = True
             if npf:
                 self._seq.latent_attention_mfma(o_lat, qc, q_abs, q, proj, meta.positions, cache, meta.seq_cu,
@@ -354,6 +362,9 @@ class ReferenceOps:
                          gate_off, scale, window):
         ref.latent_attention(o_lat, q_abs, q, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, inv_freq,
                              heads, dim, rot_dim, kv_rank, gate_off, scale, window)
+
+    def latent_query_in_place(self, dtype, kv_rank, rot_dim) -> bool:
+        return False
 
     def mingru_scan(self, y, state, proj, b_z, b_x, meta):
         ref.mingru_scan(y, state, proj, b_z, b_x, meta.seq_cu, meta.seq_ctx, meta.seq_state)
