@@ -27,7 +27,7 @@ def kesirax_config(name, s):
     attn = LatentAttentionSpec(heads=s["heads"], dim=128, rot_dim=64, vdim=128, q_rank=s["width"] // 2,
                                kv_rank=512, scale=192 ** -0.5, window=s["window"], rot_base=10000.0)
     ff = TableMoESpec(experts=s["experts"], top=s["top"], ff=s["ff"])
-    layers = tuple(HybridLayerSpec(m, ff) for m in (MinGRUSpec(s["gru"]), attn, attn, MinGRUSpec(s["gru"])))
+    layers = tuple(HybridLayerSpec(m, ff) for m in (attn, MinGRUSpec(s["gru"]), attn, MinGRUSpec(s["gru"])))
     return HybridConfig(name=f"kesirax-{name}", hidden_size=s["width"], vocab_size=s["vocab"], layers=layers,
                         norm_groups=4, max_position_embeddings=16384, eos_token_id=(2,), bos_token_id=1)
 

@@ -719,7 +719,7 @@ PRESETS.update({
     "tiny-kesirax": _mini_kesirax("tiny-kesirax", 64, 320,
                                   dict(heads=3, dim=16, rot_dim=8, vdim=24, q_rank=40, kv_rank=32, scale=24 ** -0.5,
                                        window=24, rot_base=10000.0),
-                                  48, dict(experts=4, top=2, ff=40), "gaag", loop=(1, 3, 2), groups=4),
+                                  48, dict(experts=4, top=2, ff=40), "agga", loop=(1, 3, 2), groups=4),
     # GPU-test size
     "small-kesirax": _mini_kesirax("small-kesirax", 512, 1024,
                                    dict(heads=8, dim=64, rot_dim=32, vdim=64, q_rank=192, kv_rank=128,

@@ -140,7 +140,7 @@ def moe(experts=4, top=2, ff=12):
     return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
 
 
-def make_config(layers, width=32, vocab=96, loop=(0, 0, 1), groups=2, logit_scale=0.5, eps=1e-6):
+def make_config(layers, width=32, vocab=96, loop=(0, 0, 1), groups=4, logit_scale=0.75, eps=1e-6):
     return {"architecture": "Kesirax", "layers": layers, "logit_scale": logit_scale,
             "loop": {"start": loop[0], "stop": loop[1], "times": loop[2]},
             "norm": {"eps": eps, "groups": groups}, "vocab": vocab, "width": width}

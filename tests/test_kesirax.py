@@ -41,8 +41,8 @@ def tokens(n, vocab, seed):
 
 def base_config(**kw):
     f = O.moe()
-    layers = [O.gru_layer(mlp=f), O.attn_layer(mlp=f), O.attn_layer(window=9, mlp=f), O.gru_layer(width=40, mlp=f)]
-    return O.make_config(layers, loop=(0, 3, 2), **kw)
+    layers = [O.attn_layer(mlp=f), O.gru_layer(mlp=f), O.gru_layer(width=40, mlp=f), O.attn_layer(window=9, mlp=f)]
+    return O.make_config(layers, loop=(1, 3, 2), **kw)
 
 
 def session(tmp_path, cfg, W, target, max_tokens=512, name="m"):
@@ -195,7 +195,7 @@ def test_prefill_and_long_decoding(tmp_path, target):
     check_all(replay(sess, portions(toks, [len(toks)])), "a", ref, TOL[target[1]])   # the whole prompt at once
     for got, want in zip(model.capture, streams):                                    # the stream after every layer run
         assert rel_err(got, want) < TOL[target[1]]
-    assert len(model.capture) == len(streams) == 7
+    assert len(model.capture) == len(streams) == len(O.layer_runs(cfg)) == 6
     model.capture = None
     # a short prompt, then 60 tokens one by one: the windows (6 and 9) pass over decoded tokens many times
     check_all(replay(sess, portions(toks, [10])), "a", ref, TOL[target[1]])
