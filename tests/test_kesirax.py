@@ -105,7 +105,8 @@ def one_seq_meta(T, dev, start=0, block_size=4, slot=0, perm_seed=0, total=160):
 
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("shape", [dict(), dict(heads=5, dim=16, rot_dim=8, vdim=12, q_rank=20, kv_rank=72, window=0),
-                                   dict(heads=1, rot_dim=8, rot_dims=4, window=3), dict(heads=18, window=70)])
+                                   dict(heads=1, rot_dim=8, rot_dims=4, window=3), dict(heads=18, window=70),
+                                   dict(heads=3, rot_dim=64, kv_rank=1024, window=11), dict(heads=70, kv_rank=264)])
 def test_latent_attention_alone(target, shape):
     dev, dt = torch.device(target[0]), getattr(torch, target[1])
     l = O.attn_layer(**shape)
