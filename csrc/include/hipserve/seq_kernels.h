@@ -52,4 +52,48 @@ void launch_mingru_scan(void* y, float* state, const void* proj, const float* b_
 void launch_expert_gemm(void* out, const void* x, long x_ld, const void* w, const int* slots, const int* tile_expert,
                         int ntiles_cap, int tile, int gather_k, int N, int K, bool relu2, bool f32, hipStream_t s);
 
+// Window attention on a paged cache [blocks, block_size, kv_heads * dim | kv_heads * vdim] (window_attention.hip).
+// attn_prepare: per row of proj = [q | k | v | ...]: optional whole-projection RMS norm of q and k (q_norm /
+// k_norm null: none), rotate-half rotation of the first 2 * nfreq dims per head, optional per-head unit-rms
+// values; q in place, k / v into cache row slots[t] (>= 0).
+void launch_attn_prepare(void* proj, long ld, void* cache, const long* positions, const long* slots,
+                         const float* inv_freq, int nfreq, int T, int heads, int kv_heads, int dim, int vdim,
+                         const float* q_norm, const float* k_norm, bool v_norm, float eps, bool f32, hipStream_t s);
+// Sequences seq0 .. seq1-1 of the step, `tq` tokens per workgroup: keys 0 <= pos - j < window (0: all),
+// weights exp(s_j) / (sink + sum exp), head output times sigmoid(proj[t, gate_off + h]) (gate_off >= 0) and
+// out_scale into out[t * out_ld + h * vdim ..].
+int window_attention_max_vdim();
+void launch_window_attention(void* out, long out_ld, const void* proj, long proj_ld, const void* cache, int block_size,
+                             const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0, int seq1,
+                             int rows_bound, int tq, int heads, int kv_heads, int dim, int vdim, int gate_off,
+                             float scale, int window, bool sink, float out_scale, bool f32, hipStream_t s);
+
+// bf16 on the matrix cores (window_attention_mfma.hip): 64 (token, head) rows of one key/value head per
+// workgroup, 32-key tiles. nparts > 1 (rows of one token each, rows_bound of them from batch row row_base on):
+// the keys are split into runs of part_keys (a multiple of 32) over ws_acc [nparts, heads, rows_bound, vdim] /
+// ws_ml [.., 2] and merged. out_off: element offset of `out` in its allocation (alignment of the stores).
+bool window_attention_mfma_ok(int dim, int vdim, long out_ld, long out_off);
+void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long proj_ld, const void* cache,
+                                  int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
+                                  int bt_width, int seq0, int seq1, int rows_bound, int heads, int kv_heads, int dim,
+                                  int vdim, int gate_off, float scale, int window, bool sink, float out_scale,
+                                  int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base,
+                                  hipStream_t s);
+
+// Delta-rule recurrences over state slots (delta_scan.hip). scratch: fp32, T * (2 * kv_heads * dim +
+// 2 * heads * vdim + 2 * heads) floats for the gated rule, T * 4 * heads * dim for the generalized one.
+int delta_max_dim();
+int delta_max_taps();
+void launch_gated_delta(void* y, float* S, float* conv_state, const void* proj, long ld, const float* conv_w,
+                        const float* a_log, const float* dt_bias, const float* norm_w, const int* seq_cu,
+                        const int* seq_ctx, const int* seq_state, int nseq, int T, float* scratch, int heads,
+                        int kv_heads, int dim, int vdim, int taps, float eps, bool f32, hipStream_t s);
+void launch_delta_rule(void* out, long out_ld, float* S, const void* proj, long ld, const float* wl, const float* a_b,
+                       const float* w0, const float* norm_w, const int* seq_cu, const int* seq_ctx,
+                       const int* seq_state, int nseq, int T, float* scratch, int heads, int dim, float eps,
+                       float out_scale, bool f32, hipStream_t s);
+// kind 0: tanh; 1: c0 z^2 + z/2 (z > 0), c1 (exp(z) - 1 - z) + z/2 (z <= 0).
+void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,
+                       float c1, bool f32, hipStream_t s);
+
 }  // namespace hipserve

@@ -1,0 +1,513 @@
+// Delta-rule recurrences over per-sequence state slots, fp32 state [slots, heads, key dim, value dim].
+//
+// gated delta rule (per head, one decay g and one write strength beta per token):
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// generalized delta rule (per head, decay w and removal rate a per key channel, unit key u):
+//   S <- diag(w) S - (a * u)(u^T S) + k v^T  (both terms read the old S);  o = S^T r
+//
+// Both scans keep a COLUMN of the state (all key channels of one value channel) in the registers
+// of the 16 lanes of a DPP row, dim / 16 key channels each, so a product with the state is a few
+// multiply-adds per lane and a four-step DPP sum; the per-token vectors shared by all columns (k, q / w, a u,
+// u, k, r) are staged through LDS a few tokens at a time. A step that starts at position 0 starts from a zero state.
+//
+// The prepare kernels compute what enters the recurrences in fp32: the short causal convolution
+// (+ SiLU) from the step's rows and the sequence's last taps - 1 inputs, unit vectors, sigmoid /
+// softplus / exp of the decays and rates. head_norm_gate finishes both: per-head RMS norm of the
+// read-out, weight, SiLU or sigmoid gate, optional scale.
+#include "seq_common.h"
+#include "hipserve/seq_kernels.h"
+
+namespace hipserve {
+namespace {
+
+HS_DEVICE float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+HS_DEVICE int find_seq(const int* __restrict__ seq_cu, int nseq, int row) {
+  for (int s = 0; s < nseq; ++s)
+    if (row < seq_cu[s + 1]) return row >= seq_cu[s] ? s : -1;
+  return -1;
+}
+
+// proj rows = [q | k | v | beta | decay | gate]; C = conv channels (q, k, v). One workgroup per token.
+//   qk[t] = [unit(silu(conv q)) * dim^-1/2 | unit(silu(conv k))]  per head,  vv[t] = silu(conv v),
+//   bg[t] = [beta (heads) | g (heads)].
+template <typename T>
+__global__ __launch_bounds__(256) void gated_delta_prepare_kernel(
+    float* __restrict__ qk, float* __restrict__ vv, float* __restrict__ bg, const T* __restrict__ proj, long ld,
+    const float* __restrict__ conv_state, const float* __restrict__ conv_w, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx,
+    const int* __restrict__ seq_state, int nseq, int heads, int kv_heads, int dim, int vdim, int taps) {
+  extern __shared__ float xs[];  // [C] convolved + SiLU
+  const int t = blockIdx.x;
+  const int s = find_seq(seq_cu, nseq, t);
+  if (s < 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0;
+  const bool carried = seq_ctx[s] - n > 0;
+  const int nqk = kv_heads * dim, C = 2 * nqk + heads * vdim, hist = taps - 1;
+  const float* cs = conv_state + (long)seq_state[s] * max(hist, 1) * C;
+  for (int c = tid; c < C; c += 256) {
+    float a = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int r = t - hist + j;  // batch row of the tap's input
+      float x;
+      if (r >= r0) x = ldf<T>(proj, (long)r * ld + c);
+      else x = carried ? cs[(long)(hist + r - r0) * C + c] : 0.f;
+      a = __builtin_fmaf(conv_w[(long)c * taps + j], x, a);
+    }
+    xs[c] = a * sigmoid_f(a);
+  }
+  __syncthreads();
+  for (int h = wave; h < 2 * kv_heads; h += 4) {  // unit q heads, then unit k heads
+    float a = 0.f;
+    for (int e = lane; e < dim; e += 64) { const float v = xs[h * dim + e]; a += v * v; }
+    float inv = 1.f / sqrtf(wave_sum(a) + 1e-6f);
+    if (h < kv_heads) inv *= 1.f / sqrtf((float)dim);
+    for (int e = lane; e < dim; e += 64) qk[(long)t * 2 * nqk + h * dim + e] = xs[h * dim + e] * inv;
+  }
+  const int nv = heads * vdim;
+  for (int e = tid; e < nv; e += 256) vv[(long)t * nv + e] = xs[2 * nqk + e];
+  for (int h = tid; h < heads; h += 256) {
+    const T* p = proj + (long)t * ld + C;
+    bg[(long)t * 2 * heads + h] = sigmoid_f(ldf<T>(p, h));
+    bg[(long)t * 2 * heads + heads + h] = expf(-expf(a_log[h]) * softplus_f(ldf<T>(p, heads + h) + dt_bias[h]));
+  }
+}
+
+// The last taps - 1 conv inputs of every sequence into its slot (after the prepare kernel has read the old ones).
+constexpr int kMaxHist = 15;
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    float* __restrict__ conv_state, const T* __restrict__ proj, long ld, const int* __restrict__ seq_cu,
+    const int* __restrict__ seq_ctx, const int* __restrict__ seq_state, int C, int taps) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0, hist = taps - 1;
+  if (c >= C || n <= 0 || hist <= 0) return;
+  const bool carried = seq_ctx[s] - n > 0;
+  float* cs = conv_state + (long)seq_state[s] * hist * C;
+  float keep[kMaxHist];
+#pragma unroll
+  for (int i = 0; i < kMaxHist; ++i) {
+    if (i < hist) {
+      const int j = n - hist + i;  // row of the step, or (negative) one of the old inputs
+      keep[i] = j >= 0 ? ldf<T>(proj, (long)(r0 + j) * ld + c) : (carried ? cs[(long)(hist + j) * C + c] : 0.f);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxHist; ++i)
+    if (i < hist) cs[(long)i * C + c] = keep[i];
+}
+
+constexpr int kTB = 8;     // tokens staged at a time
+constexpr int kSeg = 16;   // lanes that share a state column (one DPP row)
+constexpr int kCV = 1;     // state columns per lane (2: half the waves, each twice as long; measured slower)
+constexpr int kScanThreads = 256;
+static_assert(kCV <= 2, "the read-out store below picks outs[0] / outs[1] by lane");
+constexpr int kCols = kScanThreads / kSeg * kCV;  // state columns per workgroup
+
+// Sum over the 16 lanes of a DPP row; every lane of the row gets it.
+HS_DEVICE float row_sum(float v) {
+  v = dpp_step<0xB1, 0xf, false>(v);   // quad_perm [1, 0, 3, 2]
+  v = dpp_step<0x4E, 0xf, false>(v);   // quad_perm [2, 3, 0, 1]
+  v = dpp_step<0x141, 0xf, false>(v);  // row_half_mirror
+  return dpp_step<0x140, 0xf, false>(v);  // row_mirror
+}
+
+// grid (heads, ceil(vdim / kCols), sequences), four waves: the step's first sequences (its prompt portions, the
+// long ones) are dispatched first and spread over the CUs before the one-token sequences fill in. A state column (one value channel) is held by the 16
+// lanes of a DPP row, DS key channels each (dim <= 16 DS; the padding rows stay zero): a product with the
+// state is DS multiply-adds per lane and four DPP steps, so the chain from one token to the next is short.
+// Every lane row holds kCV columns (independent chains that fill each other's stalls and share the LDS reads
+// of the per-token vectors, which bound the kernel otherwise); the waves share the staging.
+template <int DS>
+__global__ __launch_bounds__(kScanThreads) void gated_delta_scan_kernel(
+    float* __restrict__ o, float* __restrict__ S, const float* __restrict__ qk, const float* __restrict__ vv,
+    const float* __restrict__ bg, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx,
+    const int* __restrict__ seq_state, int heads, int kv_heads, int dim, int vdim) {
+  constexpr int DP = kSeg * DS;
+  __shared__ __attribute__((aligned(16))) float sq[kTB][DP], sk[kTB][DP];
+  __shared__ float sb[kTB][2];
+  const int s = blockIdx.z, h = blockIdx.x, zb = blockIdx.y, tid = threadIdx.x;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0;
+  if (n <= 0) return;
+  const int seg = tid & (kSeg - 1), k0 = seg * DS;
+  const int v0 = zb * kCols + (tid / kSeg) * kCV;   // this lane row's first column
+  const int kh = h / (heads / kv_heads), nqk = kv_heads * dim, nv = heads * vdim;
+  float* Sp = S + (((long)seq_state[s] * heads + h) * dim) * vdim;
+  const bool carried = seq_ctx[s] - n > 0;
+  float st[kCV][DS];
+#pragma unroll
+  for (int cv = 0; cv < kCV; ++cv)
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      st[cv][i] = (carried && v0 + cv < vdim && k0 + i < dim) ? Sp[(long)(k0 + i) * vdim + v0 + cv] : 0.f;
+  // the next batch of tokens is loaded into registers while this batch is computed
+  constexpr int kLd = (kTB * DP + kScanThreads - 1) / kScanThreads;
+  float rq[kLd], rk[kLd], rv[kTB][kCV], rb = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = min(kTB, n - t0);
+#pragma unroll
+    for (int it = 0; it < kLd; ++it) {
+      const int i = it * kScanThreads + tid;
+      const int tt = i / DP, k = i % DP;
+      const long row = (long)(r0 + t0 + tt) * 2 * nqk;
+      const bool in = tt < nt && k < dim;
+      rq[it] = in ? qk[row + kh * dim + k] : 0.f;
+      rk[it] = in ? qk[row + nqk + kh * dim + k] : 0.f;
+    }
+    if (tid < 2 * nt) rb = bg[(long)(r0 + t0 + (tid >> 1)) * 2 * heads + (tid & 1) * heads + h];
+#pragma unroll
+    for (int tt = 0; tt < kTB; ++tt)
+#pragma unroll
+      for (int cv = 0; cv < kCV; ++cv)
+        rv[tt][cv] = (tt < nt && v0 + cv < vdim) ? vv[(long)(r0 + t0 + tt) * nv + h * vdim + v0 + cv] : 0.f;
+  };
+  float* po = o + (long)r0 * nv + h * vdim + v0 + seg;
+  fetch(0);
+  for (int t0 = 0; t0 < n; t0 += kTB) {
+    const int nt = min(kTB, n - t0);
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kLd; ++it) {
+      const int i = it * kScanThreads + tid;
+      if (i < kTB * DP) {
+        sq[i / DP][i % DP] = rq[it];
+        sk[i / DP][i % DP] = rk[it];
+      }
+    }
+    if (tid < 2 * kTB) sb[tid >> 1][tid & 1] = rb;
+    float val[kTB][kCV];
+#pragma unroll
+    for (int tt = 0; tt < kTB; ++tt)
+#pragma unroll
+      for (int cv = 0; cv < kCV; ++cv) val[tt][cv] = rv[tt][cv];
+    __syncthreads();
+    if (t0 + kTB < n) fetch(t0 + kTB);
+#pragma unroll
+    for (int tt = 0; tt < kTB; ++tt) {
+      if (tt < nt) {
+        const float beta = sb[tt][0], g = sb[tt][1];
+        float kk[DS], qq[DS];
+#pragma unroll
+        for (int i = 0; i < DS; ++i) { kk[i] = sk[tt][k0 + i]; qq[i] = sq[tt][k0 + i]; }
+        float outs[kCV];
+#pragma unroll
+        for (int cv = 0; cv < kCV; ++cv) {
+          float pred = 0.f, pred2 = 0.f;
+#pragma unroll
+          for (int i = 0; i < DS; ++i) {
+            st[cv][i] *= g;
+            if (i & 1) pred2 = __builtin_fmaf(st[cv][i], kk[i], pred2);
+            else pred = __builtin_fmaf(st[cv][i], kk[i], pred);
+          }
+          const float u = beta * (val[tt][cv] - row_sum(pred + pred2));
+          float out = 0.f, out2 = 0.f;
+#pragma unroll
+          for (int i = 0; i < DS; ++i) {
+            st[cv][i] = __builtin_fmaf(kk[i], u, st[cv][i]);
+            if (i & 1) out2 = __builtin_fmaf(st[cv][i], qq[i], out2);
+            else out = __builtin_fmaf(st[cv][i], qq[i], out);
+          }
+          outs[cv] = row_sum(out + out2);
+        }
+        if (seg < kCV && v0 + seg < vdim) po[(long)(t0 + tt) * nv] = seg == 0 ? outs[0] : outs[kCV - 1];
+      }
+    }
+  }
+#pragma unroll
+  for (int cv = 0; cv < kCV; ++cv)
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      if (v0 + cv < vdim && k0 + i < dim) Sp[(long)(k0 + i) * vdim + v0 + cv] = st[cv][i];
+}
+
+// proj rows = [r | k | v | a | g | ...] (N = heads * dim each), wl = decay pre-activation (fp32 [T, N]).
+// pre[t] = [w = exp(-e^-1/2 sigmoid(wl + w0)) | a u | u] with a = sigmoid(a + a_b), u = unit(k) per head.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_rule_prepare_kernel(
+    float* __restrict__ pre, const T* __restrict__ proj, long ld, const float* __restrict__ wl,
+    const float* __restrict__ a_b, const float* __restrict__ w0, int heads, int dim) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int N = heads * dim;
+  const T* row = proj + t * ld;
+  for (int h = wave; h < heads; h += 4) {
+    float a = 0.f;
+    for (int e = lane; e < dim; e += 64) { const float v = ldf<T>(row, N + h * dim + e); a += v * v; }
+    const float inv = 1.f / sqrtf(wave_sum(a) + 1e-6f);
+    for (int e = lane; e < dim; e += 64) {
+      const int c = h * dim + e;
+      const float u = ldf<T>(row, N + c) * inv;
+      pre[t * 3 * N + c] = expf(-0.60653065971263342f * sigmoid_f(wl[t * N + c] + w0[c]));
+      pre[t * 3 * N + N + c] = sigmoid_f(ldf<T>(row, 3 * N + c) + a_b[c]) * u;
+      pre[t * 3 * N + 2 * N + c] = u;
+    }
+  }
+}
+
+template <typename T, int DS>
+__global__ __launch_bounds__(kScanThreads) void delta_rule_scan_kernel(
+    float* __restrict__ o, float* __restrict__ S, const float* __restrict__ pre, const T* __restrict__ proj, long ld,
+    const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx, const int* __restrict__ seq_state, int heads,
+    int dim) {
+  constexpr int DP = kSeg * DS, TB = kTB;
+  __shared__ __attribute__((aligned(16))) float sv[TB][5][DP];  // w, a u, u, k, r (zero past dim)
+  const int s = blockIdx.z, h = blockIdx.x, zb = blockIdx.y, tid = threadIdx.x;
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0;
+  if (n <= 0) return;
+  const int seg = tid & (kSeg - 1), k0 = seg * DS;
+  const int v0 = zb * kCols + (tid / kSeg) * kCV;   // this lane row's first column
+  const int N = heads * dim;
+  float* Sp = S + (((long)seq_state[s] * heads + h) * dim) * dim;
+  const bool carried = seq_ctx[s] - n > 0;
+  float st[kCV][DS];
+#pragma unroll
+  for (int cv = 0; cv < kCV; ++cv)
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      st[cv][i] = (carried && v0 + cv < dim && k0 + i < dim) ? Sp[(long)(k0 + i) * dim + v0 + cv] : 0.f;
+  // the next batch of tokens is loaded into registers while this batch is computed
+  constexpr int kLd = (TB * DP + kScanThreads - 1) / kScanThreads;
+  float rg[5][kLd], rv[TB][kCV];
+  auto fetch = [&](int t0) {
+    const int nt = min(TB, n - t0);
+#pragma unroll
+    for (int it = 0; it < kLd; ++it) {
+      const int i = it * kScanThreads + tid;
+      const int tt = i / DP, k = i % DP;
+      const long row = r0 + t0 + tt;
+      const int c = h * dim + k;
+      const bool in = tt < nt && k < dim;
+      rg[0][it] = in ? pre[row * 3 * N + c] : 0.f;
+      rg[1][it] = in ? pre[row * 3 * N + N + c] : 0.f;
+      rg[2][it] = in ? pre[row * 3 * N + 2 * N + c] : 0.f;
+      rg[3][it] = in ? ldf<T>(proj, row * ld + N + c) : 0.f;
+      rg[4][it] = in ? ldf<T>(proj, row * ld + c) : 0.f;
+    }
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt)
+#pragma unroll
+      for (int cv = 0; cv < kCV; ++cv)
+        rv[tt][cv] = (tt < nt && v0 + cv < dim) ? ldf<T>(proj, (long)(r0 + t0 + tt) * ld + 2 * N + h * dim + v0 + cv) : 0.f;
+  };
+  float* po = o + (long)r0 * N + h * dim + v0 + seg;
+  fetch(0);
+  for (int t0 = 0; t0 < n; t0 += TB) {
+    const int nt = min(TB, n - t0);
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kLd; ++it) {
+      const int i = it * kScanThreads + tid;
+      if (i < TB * DP) {
+#pragma unroll
+        for (int j = 0; j < 5; ++j) sv[i / DP][j][i % DP] = rg[j][it];
+      }
+    }
+    float val[TB][kCV];
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt)
+#pragma unroll
+      for (int cv = 0; cv < kCV; ++cv) val[tt][cv] = rv[tt][cv];
+    __syncthreads();
+    if (t0 + TB < n) fetch(t0 + TB);
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      if (tt < nt) {
+        float w[DS], au[DS], uu[DS], kk[DS], rr[DS];
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+          w[i] = sv[tt][0][k0 + i]; au[i] = sv[tt][1][k0 + i]; uu[i] = sv[tt][2][k0 + i];
+          kk[i] = sv[tt][3][k0 + i]; rr[i] = sv[tt][4][k0 + i];
+        }
+        float outs[kCV];
+#pragma unroll
+        for (int cv = 0; cv < kCV; ++cv) {
+          float us = 0.f, us2 = 0.f;
+#pragma unroll
+          for (int i = 0; i < DS; ++i) {
+            if (i & 1) us2 = __builtin_fmaf(uu[i], st[cv][i], us2);
+            else us = __builtin_fmaf(uu[i], st[cv][i], us);
+          }
+          us = row_sum(us + us2);
+          float out = 0.f, out2 = 0.f;
+#pragma unroll
+          for (int i = 0; i < DS; ++i) {
+            st[cv][i] = w[i] * st[cv][i] - au[i] * us + kk[i] * val[tt][cv];
+            if (i & 1) out2 = __builtin_fmaf(st[cv][i], rr[i], out2);
+            else out = __builtin_fmaf(st[cv][i], rr[i], out);
+          }
+          outs[cv] = row_sum(out + out2);
+        }
+        if (seg < kCV && v0 + seg < dim) po[(long)(t0 + tt) * N] = seg == 0 ? outs[0] : outs[kCV - 1];
+      }
+    }
+  }
+#pragma unroll
+  for (int cv = 0; cv < kCV; ++cv)
+#pragma unroll
+    for (int i = 0; i < DS; ++i)
+      if (v0 + cv < dim && k0 + i < dim) Sp[(long)(k0 + i) * dim + v0 + cv] = st[cv][i];
+}
+
+// One wave per (token, head): out = o / rms(o) * w[head * w_stride + e] * act(gate) * scale.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(
+    T* __restrict__ out, long out_ld, const float* __restrict__ o, const T* __restrict__ proj, long ld, int gate_off,
+    const float* __restrict__ w, int w_stride, int rows, int heads, int vdim, float eps, bool silu, float scale) {
+  const long idx = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (idx >= (long)rows * heads) return;
+  const long t = idx / heads;
+  const int h = idx % heads;
+  const float* src = o + (t * heads + h) * vdim;
+  float a = 0.f;
+  for (int e = lane; e < vdim; e += 64) { const float x = src[e]; a += x * x; }
+  const float inv = scale / sqrtf(wave_sum(a) / (float)vdim + eps);
+  const T* gate = proj + t * ld + gate_off + (long)h * vdim;
+  for (int e = lane; e < vdim; e += 64) {
+    const float gp = ldf<T>(gate, e);
+    const float gv = silu ? gp * sigmoid_f(gp) : sigmoid_f(gp);
+    stf<T>(out, t * out_ld + (long)h * vdim + e, src[e] * inv * w[h * w_stride + e] * gv);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ out, long out_ld, const T* __restrict__ x,
+                                                         long x_ld, int cols, int kind, float c0, float c1) {
+  const long t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= cols) return;
+  const float z = ldf<T>(x, t * x_ld + c);
+  float r;
+  if (kind == 0) r = tanhf(z);
+  else r = z > 0.f ? c0 * z * z + 0.5f * z : c1 * (expm1f(z) - z) + 0.5f * z;
+  stf<T>(out, t * out_ld + c, r);
+}
+
+// bf16 rows whose length, strides and base addresses are multiples of 8 elements: 8 elements per thread.
+__global__ __launch_bounds__(256) void activation_vec_kernel(unsigned short* __restrict__ out, long out_ld,
+                                                             const unsigned short* __restrict__ x, long x_ld,
+                                                             int cols8, int kind, float c0, float c1) {
+  const long t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= cols8) return;
+  const u16x8 z8 = *reinterpret_cast<const u16x8*>(x + t * x_ld + 8 * c);
+  u16x8 r8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float z = bf16_to_f32(z8[e]);
+    float r;
+    if (kind == 0) r = tanhf(z);
+    else r = z > 0.f ? c0 * z * z + 0.5f * z : c1 * (expm1f(z) - z) + 0.5f * z;
+    r8[e] = f32_to_bf16(r);
+  }
+  *reinterpret_cast<u16x8*>(out + t * out_ld + 8 * c) = r8;
+}
+
+template <typename T>
+void head_norm_gate(void* out, long out_ld, const float* o, const void* proj, long ld, int gate_off, const float* w,
+                    int w_stride, int rows, int heads, int vdim, float eps, bool silu, float scale, hipStream_t s) {
+  const long n = (long)rows * heads;
+  head_norm_gate_kernel<T><<<(unsigned)((n + 3) / 4), 256, 0, s>>>((T*)out, out_ld, o, (const T*)proj, ld, gate_off, w,
+                                                                   w_stride, rows, heads, vdim, eps, silu, scale);
+}
+
+int ds_of(int dim) { return dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : 16; }
+
+}  // namespace
+
+int delta_max_dim() { return 256; }
+int delta_max_taps() { return kMaxHist + 1; }
+
+void launch_gated_delta(void* y, float* S, float* conv_state, const void* proj, long ld, const float* conv_w,
+                        const float* a_log, const float* dt_bias, const float* norm_w, const int* seq_cu,
+                        const int* seq_ctx, const int* seq_state, int nseq, int T, float* scratch, int heads,
+                        int kv_heads, int dim, int vdim, int taps, float eps, bool f32, hipStream_t s) {
+  if (nseq <= 0 || T <= 0) return;
+  const int nqk = kv_heads * dim, nv = heads * vdim, C = 2 * nqk + nv;
+  float* qk = scratch;                       // [T, 2 nqk]
+  float* vv = qk + (long)T * 2 * nqk;        // [T, nv]
+  float* bg = vv + (long)T * nv;             // [T, 2 heads]
+  float* o = bg + (long)T * 2 * heads;       // [T, nv]
+  const size_t smem = (size_t)C * sizeof(float);
+  dim3 ugrid(nseq, (C + 255) / 256);
+  if (f32) {
+    gated_delta_prepare_kernel<float><<<T, 256, smem, s>>>(qk, vv, bg, (const float*)proj, ld, conv_state, conv_w,
+                                                           a_log, dt_bias, seq_cu, seq_ctx, seq_state, nseq, heads,
+                                                           kv_heads, dim, vdim, taps);
+    conv_state_update_kernel<float><<<ugrid, 256, 0, s>>>(conv_state, (const float*)proj, ld, seq_cu, seq_ctx,
+                                                          seq_state, C, taps);
+  } else {
+    gated_delta_prepare_kernel<unsigned short><<<T, 256, smem, s>>>(
+        qk, vv, bg, (const unsigned short*)proj, ld, conv_state, conv_w, a_log, dt_bias, seq_cu, seq_ctx, seq_state,
+        nseq, heads, kv_heads, dim, vdim, taps);
+    conv_state_update_kernel<unsigned short><<<ugrid, 256, 0, s>>>(conv_state, (const unsigned short*)proj, ld, seq_cu,
+                                                                   seq_ctx, seq_state, C, taps);
+  }
+  dim3 grid(heads, (vdim + kCols - 1) / kCols, nseq);
+  switch (ds_of(dim)) {
+#define HS_GD(D)                                                                                                     \
+  case D:                                                                                                            \
+    gated_delta_scan_kernel<D><<<grid, kScanThreads, 0, s>>>(o, S, qk, vv, bg, seq_cu, seq_ctx, seq_state, heads, kv_heads, dim, \
+                                                   vdim);                                                            \
+    break;
+    HS_GD(1) HS_GD(2) HS_GD(4) HS_GD(8) HS_GD(16)
+#undef HS_GD
+  }
+  const int gate_off = C + 2 * heads;
+  if (f32) head_norm_gate<float>(y, nv, o, proj, ld, gate_off, norm_w, 0, T, heads, vdim, eps, true, 1.f, s);
+  else head_norm_gate<unsigned short>(y, nv, o, proj, ld, gate_off, norm_w, 0, T, heads, vdim, eps, true, 1.f, s);
+}
+
+void launch_delta_rule(void* out, long out_ld, float* S, const void* proj, long ld, const float* wl, const float* a_b,
+                       const float* w0, const float* norm_w, const int* seq_cu, const int* seq_ctx,
+                       const int* seq_state, int nseq, int T, float* scratch, int heads, int dim, float eps,
+                       float out_scale, bool f32, hipStream_t s) {
+  if (nseq <= 0 || T <= 0) return;
+  const int N = heads * dim;
+  float* pre = scratch;               // [T, 3 N]
+  float* o = pre + (long)T * 3 * N;   // [T, N]
+  dim3 grid(heads, (dim + kCols - 1) / kCols, nseq);
+  if (f32) {
+    delta_rule_prepare_kernel<float><<<T, 256, 0, s>>>(pre, (const float*)proj, ld, wl, a_b, w0, heads, dim);
+    switch (ds_of(dim)) {
+#define HS_DR(D)                                                                                                  \
+  case D:                                                                                                         \
+    delta_rule_scan_kernel<float, D><<<grid, kScanThreads, 0, s>>>(o, S, pre, (const float*)proj, ld, seq_cu, seq_ctx,      \
+                                                         seq_state, heads, dim);                                  \
+    break;
+      HS_DR(1) HS_DR(2) HS_DR(4) HS_DR(8) HS_DR(16)
+#undef HS_DR
+    }
+    head_norm_gate<float>(out, out_ld, o, proj, ld, 4 * N, norm_w, dim, T, heads, dim, eps, false, out_scale, s);
+  } else {
+    delta_rule_prepare_kernel<unsigned short><<<T, 256, 0, s>>>(pre, (const unsigned short*)proj, ld, wl, a_b, w0,
+                                                                heads, dim);
+    switch (ds_of(dim)) {
+#define HS_DR(D)                                                                                                   \
+  case D:                                                                                                          \
+    delta_rule_scan_kernel<unsigned short, D><<<grid, kScanThreads, 0, s>>>(o, S, pre, (const unsigned short*)proj, ld, seq_cu, \
+                                                                  seq_ctx, seq_state, heads, dim);                 \
+    break;
+      HS_DR(1) HS_DR(2) HS_DR(4) HS_DR(8) HS_DR(16)
+#undef HS_DR
+    }
+    head_norm_gate<unsigned short>(out, out_ld, o, proj, ld, 4 * N, norm_w, dim, T, heads, dim, eps, false, out_scale,
+                                   s);
+  }
+}
+
+void launch_activation(void* out, long out_ld, const void* x, long x_ld, int rows, int cols, int kind, float c0,
+                       float c1, bool f32, hipStream_t s) {
+  if (rows <= 0 || cols <= 0) return;
+  dim3 grid(rows, (cols + 255) / 256);
+  if (f32) activation_kernel<float><<<grid, 256, 0, s>>>((float*)out, out_ld, (const float*)x, x_ld, cols, kind, c0, c1);
+  else if (cols % 8 == 0 && out_ld % 8 == 0 && x_ld % 8 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)x % 16 == 0)
+    activation_vec_kernel<<<dim3(rows, (cols / 8 + 255) / 256), 256, 0, s>>>(
+        (unsigned short*)out, out_ld, (const unsigned short*)x, x_ld, cols / 8, kind, c0, c1);
+  else
+    activation_kernel<unsigned short><<<grid, 256, 0, s>>>((unsigned short*)out, out_ld, (const unsigned short*)x, x_ld,
+                                                           cols, kind, c0, c1);
+}
+
+}  // namespace hipserve

@@ -1,5 +1,5 @@
 // Residual update + grouped RMSNorm of the layer-list decoders, one workgroup per token row:
-//   r = residual + ls1 * mix + ls2 * (1/top) * sum_j y[pair_slot[t*top + j]] + extra     (fp32, written back)
+//   r = residual + ls1 * mix (ls1 null: 1) + ls2 * (1/top) * sum_j y[pair_slot[t*top + j]] + extra     (fp32, written back)
 //   out = r / sqrt(mean over the element's group of r^2 + eps) * w
 // The row is split into `groups` equal consecutive parts with their own mean square. The MoE
 // combine (rows of the expert-sorted y picked through pair_slot) and the embedding re-added at
@@ -26,7 +26,7 @@ __global__ __launch_bounds__(kNT) void scaled_add_group_rmsnorm_kernel(
   const float wtop = top > 0 ? 1.f / (float)top : 0.f;
   for (int e = tid; e < H; e += kNT) {
     float v = r[e];
-    if (mix != nullptr) v += ldf<T>(mix, t * H + e) * ls1[e];
+    if (mix != nullptr) v += ls1 != nullptr ? ldf<T>(mix, t * H + e) * ls1[e] : ldf<T>(mix, t * H + e);
     if (y != nullptr) {
       float f = 0.f;
       for (int j = 0; j < top; ++j) f += ldf<T>(y, (long)pair_slot[t * top + j] * H + e);

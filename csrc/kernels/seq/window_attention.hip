@@ -1,0 +1,257 @@
+// Grouped-query attention over a sliding window on a paged cache [blocks, block_size, keys | values]
+// (all key heads of a token, then all its value heads), with an optional softmax sink and an
+// optional per-head output gate.
+//
+// attn_prepare: per token, on the merged projection row [q | k | v | ...] (biases already added):
+// the optional RMS norm over the WHOLE q (and k) projection with a weight per element, the
+// rotate-half rotation of the first 2 * nfreq dims of every q / k head (angle = pos * inv_freq[i],
+// fp32), the optional division of every value head by its root mean square, q written back in
+// place, k and v into the cache row.
+//
+// window_attention: one wave per (token, query head) row; a workgroup holds `tq` tokens x the
+// query heads of ONE key/value head, so each 64-key tile is staged once for all of them. Scores:
+// lane = key, the head's key dims staged in chunks of 64 through LDS; online softmax per wave;
+// output: lane = value dim. With the sink the running (max, sum) start at (0, 1): a key of score
+// 0 without a value. Scores, softmax and accumulation are fp32 for both element types.
+#include "seq_common.h"
+#include "hipserve/seq_kernels.h"
+
+namespace hipserve {
+namespace {
+
+// One head's rotation work items: `dim - nfreq` per head; item i < nfreq is the pair (i, i + nfreq),
+// item i >= nfreq the unrotated element i + nfreq. Every element belongs to exactly one item.
+template <typename T, typename F>
+HS_DEVICE void rotate_heads(const T* __restrict__ src, int nheads, int dim, int nfreq, float pos,
+                            const float* __restrict__ inv_freq, float inv, const float* __restrict__ w, int tid,
+                            F&& store) {
+  const int per = dim - nfreq;
+  for (int it = tid; it < nheads * per; it += 256) {
+    const int h = it / per, i = it % per;
+    const int e0 = h * dim + (i < nfreq ? i : i + nfreq);
+    float a = ldf<T>(src, e0) * inv;
+    if (w != nullptr) a *= w[e0];
+    if (i < nfreq) {
+      const int e1 = e0 + nfreq;
+      float b = ldf<T>(src, e1) * inv;
+      if (w != nullptr) b *= w[e1];
+      float sn, cs;
+      sincosf(pos * inv_freq[i], &sn, &cs);
+      store(e0, a * cs - b * sn);
+      store(e1, b * cs + a * sn);
+    } else {
+      store(e0, a);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_prepare_kernel(
+    T* __restrict__ proj, long ld, T* __restrict__ cache, const long* __restrict__ positions,
+    const long* __restrict__ slots, const float* __restrict__ inv_freq, int nfreq, int heads, int kv_heads, int dim,
+    int vdim, const float* __restrict__ q_norm, const float* __restrict__ k_norm, bool v_norm, float eps) {
+  __shared__ float scratch[8];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nq = heads * dim, nk = kv_heads * dim, nv = kv_heads * vdim;
+  T* row = proj + t * ld;
+  float iq = 1.f, ik = 1.f;
+  if (q_norm != nullptr) {
+    float a = 0.f, b = 0.f;
+    for (int e = tid; e < nq; e += 256) { const float v = ldf<T>(row, e); a += v * v; }
+    for (int e = tid; e < nk; e += 256) { const float v = ldf<T>(row, nq + e); b += v * v; }
+    a = block_sum(a, scratch);
+    b = block_sum(b, scratch);
+    iq = 1.f / sqrtf(a / (float)nq + eps);
+    ik = 1.f / sqrtf(b / (float)nk + eps);
+  }
+  const float pos = (float)positions[t];
+  rotate_heads<T>(row, heads, dim, nfreq, pos, inv_freq, iq, q_norm, tid, [&](int e, float v) { stf<T>(row, e, v); });
+  const long slot = slots[t];
+  if (slot < 0) return;
+  T* dst = cache + slot * (long)(nk + nv);
+  rotate_heads<T>(row + nq, kv_heads, dim, nfreq, pos, inv_freq, ik, k_norm, tid,
+                  [&](int e, float v) { stf<T>(dst, e, v); });
+  const T* vr = row + nq + nk;
+  for (int g = wave; g < kv_heads; g += 4) {  // one wave per value head
+    float inv = 1.f;
+    if (v_norm) {
+      float a = 0.f;
+      for (int e = lane; e < vdim; e += 64) { const float v = ldf<T>(vr, g * vdim + e); a += v * v; }
+      inv = 1.f / sqrtf(wave_sum(a) / (float)vdim + eps);
+    }
+    for (int e = lane; e < vdim; e += 64) stf<T>(dst, nk + g * vdim + e, ldf<T>(vr, g * vdim + e) * inv);
+  }
+}
+
+constexpr int kKT = 64;       // keys per tile (one per lane)
+constexpr int kDC = 64;       // key / value dims per staged chunk
+constexpr int kMaxCh = 8;     // vdim <= kMaxCh * 64
+constexpr int kMaxRows = 16;  // waves per workgroup
+
+HS_DEVICE bool find_row_tile(const int* __restrict__ seq_cu, int seq0, int seq1, int tq, int wg, int& s, int& tok0) {
+  int acc = 0;
+  for (int i = seq0; i < seq1; ++i) {
+    const int n = seq_cu[i + 1] - seq_cu[i];
+    const int nt = (n + tq - 1) / tq;
+    if (wg < acc + nt) {
+      s = i;
+      tok0 = (wg - acc) * tq;
+      return true;
+    }
+    acc += nt;
+  }
+  return false;
+}
+
+// grid.y = kv_heads * hchunks: workgroup y serves query heads g * group + c * hc .. of key/value head g.
+template <typename T>
+__global__ __launch_bounds__(64 * kMaxRows) void window_attention_kernel(
+    T* __restrict__ out, long out_ld, const T* __restrict__ proj, long proj_ld, const T* __restrict__ cache,
+    int block_size, const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt,
+    int bt_width, int seq0, int seq1, int tq, int hc, int hchunks, int heads, int kv_heads, int dim, int vdim,
+    int gate_off, float scale, int window, bool sink, float out_scale) {
+  extern __shared__ float sm[];
+  const int nrows = blockDim.x >> 6;
+  long* krow = reinterpret_cast<long*>(sm);        // [kKT] cache row offsets (elements), -1 = no key
+  float* qs = sm + 2 * kKT;                        // [nrows][dim]
+  float* kc = qs + nrows * dim;                    // [kKT][kDC + 1]
+  float* ps = kc + kKT * (kDC + 1);                // [nrows][kKT]
+  int s, tok0;
+  if (!find_row_tile(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int group = heads / kv_heads;
+  const int g = blockIdx.y / hchunks, h0 = (blockIdx.y % hchunks) * hc;
+  const int nh = min(hc, group - h0);
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0, ctx = seq_ctx[s];
+  const int ntok = min(tq, n - tok0);
+  const int wt = wave / hc, wh = wave % hc;
+  const bool active = wt < ntok && wh < nh;
+  const int trow = r0 + tok0 + (active ? wt : 0);
+  const int head = g * group + h0 + (active ? wh : 0);
+  const int pos = ctx - n + tok0 + (active ? wt : 0);
+  const long Dc = (long)kv_heads * (dim + vdim);
+  const long koff = (long)g * dim, voff = (long)kv_heads * dim + (long)g * vdim;
+  if (active) {
+    const T* q = proj + (long)trow * proj_ld + (long)head * dim;
+    for (int e = lane; e < dim; e += 64) qs[wave * dim + e] = ldf<T>(q, e);
+  }
+  const int p_first = ctx - n + tok0, p_last = p_first + ntok - 1;
+  const int lo = window > 0 ? max(0, p_first - window + 1) : 0;
+  const int my_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float acc[kMaxCh];
+#pragma unroll
+  for (int c = 0; c < kMaxCh; ++c) acc[c] = 0.f;
+  const int nkc = (dim + kDC - 1) / kDC, nvc = (vdim + kDC - 1) / kDC;
+  for (int j0 = lo; j0 <= p_last; j0 += kKT) {
+    __syncthreads();  // the previous tile's chunk reads are done (and qs is staged, the first time)
+    if (tid < kKT) {
+      const int j = j0 + tid;
+      krow[tid] = j <= p_last ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dc
+                              : -1;
+    }
+    float sc = 0.f;
+    for (int c = 0; c < nkc; ++c) {
+      __syncthreads();
+      const int d0 = c * kDC, dn = min(kDC, dim - d0);
+      for (int idx = tid; idx < kKT * kDC; idx += blockDim.x) {
+        const int k = idx / kDC, d = idx % kDC;
+        const long kr = krow[k];
+        kc[k * (kDC + 1) + d] = (kr >= 0 && d < dn) ? ldf<T>(cache, kr + koff + d0 + d) : 0.f;
+      }
+      __syncthreads();
+      if (active) {
+        const float* qv = qs + wave * dim + d0;
+        const float* kv = kc + lane * (kDC + 1);
+        for (int d = 0; d < dn; ++d) sc = __builtin_fmaf(qv[d], kv[d], sc);
+      }
+    }
+    const int j = j0 + lane;
+    const bool vis = active && j <= pos && j >= my_lo;
+    sc = vis ? sc * scale : -INFINITY;
+    const float tmax = wave_max(sc);
+    float p = 0.f, alpha = 1.f;
+    if (tmax > -INFINITY) {  // wave-uniform: some key of the tile is visible to this row
+      const float mn = fmaxf(m, tmax);
+      alpha = expf(m - mn);   // m = -inf the first time (no sink): 0
+      p = vis ? expf(sc - mn) : 0.f;
+      l = l * alpha + wave_sum(p);
+      m = mn;
+    }
+    ps[wave * kKT + lane] = p;
+    for (int c = 0; c < nvc; ++c) {
+      __syncthreads();
+      const int d0 = c * kDC, dn = min(kDC, vdim - d0);
+      for (int idx = tid; idx < kKT * kDC; idx += blockDim.x) {
+        const int k = idx / kDC, d = idx % kDC;
+        const long kr = krow[k];
+        kc[k * (kDC + 1) + d] = (kr >= 0 && d < dn) ? ldf<T>(cache, kr + voff + d0 + d) : 0.f;
+      }
+      __syncthreads();
+      float o = 0.f;
+      const float* pv = ps + wave * kKT;
+      for (int k = 0; k < kKT; ++k) o = __builtin_fmaf(pv[k], kc[k * (kDC + 1) + lane], o);
+#pragma unroll
+      for (int cc = 0; cc < kMaxCh; ++cc)
+        if (cc == c) acc[cc] = acc[cc] * alpha + o;
+    }
+  }
+  if (!active) return;
+  float f = out_scale;
+  if (gate_off >= 0) f *= sigmoid_f(ldf<T>(proj, (long)trow * proj_ld + gate_off + head));
+  const float inv = l > 0.f ? f / l : 0.f;
+  T* dst = out + (long)trow * out_ld + (long)head * vdim;
+#pragma unroll
+  for (int c = 0; c < kMaxCh; ++c) {
+    const int e = c * kDC + lane;
+    if (c < nvc && e < vdim) stf<T>(dst, e, acc[c] * inv);
+  }
+}
+
+}  // namespace
+
+void launch_attn_prepare(void* proj, long ld, void* cache, const long* positions, const long* slots,
+                         const float* inv_freq, int nfreq, int T, int heads, int kv_heads, int dim, int vdim,
+                         const float* q_norm, const float* k_norm, bool v_norm, float eps, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    attn_prepare_kernel<float><<<T, 256, 0, s>>>((float*)proj, ld, (float*)cache, positions, slots, inv_freq, nfreq,
+                                                 heads, kv_heads, dim, vdim, q_norm, k_norm, v_norm, eps);
+  else
+    attn_prepare_kernel<unsigned short><<<T, 256, 0, s>>>((unsigned short*)proj, ld, (unsigned short*)cache, positions,
+                                                          slots, inv_freq, nfreq, heads, kv_heads, dim, vdim, q_norm,
+                                                          k_norm, v_norm, eps);
+}
+
+int window_attention_max_vdim() { return kMaxCh * kDC; }
+
+void launch_window_attention(void* out, long out_ld, const void* proj, long proj_ld, const void* cache, int block_size,
+                             const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0, int seq1,
+                             int rows_bound, int tq, int heads, int kv_heads, int dim, int vdim, int gate_off,
+                             float scale, int window, bool sink, float out_scale, bool f32, hipStream_t s) {
+  if (seq1 <= seq0 || rows_bound <= 0) return;
+  const int group = heads / kv_heads;
+  auto lds = [&](int rows) {
+    return ((size_t)rows * dim + kKT * (kDC + 1) + (size_t)rows * kKT) * sizeof(float) + kKT * sizeof(long);
+  };
+  while (tq > 1 && tq > kMaxRows) tq /= 2;
+  int hc = min(group, kMaxRows / tq);
+  while (lds(tq * hc) > 60 * 1024 && tq > 1) { tq /= 2; hc = min(group, kMaxRows / tq); }
+  while (lds(tq * hc) > 60 * 1024 && hc > 1) hc /= 2;
+  const int hchunks = (group + hc - 1) / hc;
+  const int nrows = tq * hc;
+  dim3 grid(rows_bound / tq + (seq1 - seq0), kv_heads * hchunks), block(64 * nrows);
+  const size_t smem = lds(nrows);
+  if (f32)
+    window_attention_kernel<float><<<grid, block, smem, s>>>(
+        (float*)out, out_ld, (const float*)proj, proj_ld, (const float*)cache, block_size, seq_cu, seq_ctx, seq_bt,
+        bt_width, seq0, seq1, tq, hc, hchunks, heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale);
+  else
+    window_attention_kernel<unsigned short><<<grid, block, smem, s>>>(
+        (unsigned short*)out, out_ld, (const unsigned short*)proj, proj_ld, (const unsigned short*)cache, block_size,
+        seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, hchunks, heads, kv_heads, dim, vdim, gate_off, scale,
+        window, sink, out_scale);
+}
+
+}  // namespace hipserve

@@ -1,0 +1,326 @@
+// Window attention on the matrix cores (bf16 activations and cache), same contract as the generic
+// kernel of window_attention.hip: paged cache rows [all key heads | all value heads], sliding
+// window, optional softmax sink, optional per-head sigmoid output gate, output scale.
+//
+// A workgroup (4 waves) owns 64 or 128 (token, query head) rows of ONE key/value head: consecutive
+// tokens of one sequence x the query heads of the group, so all rows share one run of keys and a
+// key / value tile is staged once for the whole group. A wave owns its 16 or 32 rows from the scores
+// to the output, so the weights P never leave its registers. Per 32-key tile:
+//   1. the head's key rows go to LDS row-major, its value rows TRANSPOSED (value dim major, the 32
+//      keys of a row permuted into the order the score registers hold them, the row's four 8-key
+//      chunks XOR-swizzled by the row index so the 2-byte transposing stores spread over the
+//      banks), loaded one tile ahead;
+//   2. S^T = K . Q^T per wave (mfma_f32_16x16x32_bf16, Q operands in registers): lane (c, g) holds
+//      the scores of row c against keys 16 nt + 4 g + i;
+//   3. masked online softmax in fp32 (log2 domain) in registers (a row's scores sit in four lanes); the
+//      sink starts the running (max, sum) at (0, 1);
+//   4. O^T += V^T . P^T: the MFMA's k slot (g, e) stands for key 16 (e / 4) + 4 g + e % 4, which is
+//      both where P's registers already are and one 16-byte read of the transposed value tile.
+// Rows with few tokens and many keys (decode) split their keys over grid.z; the runs' unnormalised
+// outputs and (max, sum) are merged by window_attention_reduce.
+#include "seq_common.h"
+#include "hipserve/seq_kernels.h"
+
+namespace hipserve {
+namespace {
+
+constexpr int kKeys = 32;   // keys per tile
+constexpr int kVLd = 40;    // transposed value tile: row stride in elements (32 keys + pad, 16-byte aligned rows)
+constexpr int kNW = 4, kRows = 16 * kNW /* x MT */, kThreads = 64 * kNW, kFT = kThreads / kKeys;
+
+template <int KS> struct KLd { static constexpr int v = KS * 32 + 8; };
+
+HS_DEVICE bool find_tile_rows(const int* __restrict__ seq_cu, int seq0, int seq1, int tq, int wg, int& s, int& tok0) {
+  int acc = 0;
+  for (int i = seq0; i < seq1; ++i) {
+    const int n = seq_cu[i + 1] - seq_cu[i];
+    const int nt = (n + tq - 1) / tq;
+    if (wg < acc + nt) {
+      s = i;
+      tok0 = (wg - acc) * tq;
+      return true;
+    }
+    acc += nt;
+  }
+  return false;
+}
+
+// KS: 32-dim steps of a key head (dim <= 32 KS); NV: 16-dim tiles of a value head (vdim <= 16 NV); MT: 16-row
+// tiles per wave (a workgroup owns 64 MT rows; every key / value operand read from LDS feeds MT MFMAs).
+template <int KS, int NV, int MT>
+__global__ __launch_bounds__(kThreads, 2) void window_attention_mfma_kernel(
+    unsigned short* __restrict__ out, long out_ld, const unsigned short* __restrict__ proj, long proj_ld,
+    const unsigned short* __restrict__ cache, int block_size, const int* __restrict__ seq_cu,
+    const int* __restrict__ seq_ctx, const int* __restrict__ seq_bt, int bt_width, int seq0, int seq1, int tq, int hc,
+    int hchunks, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale, int window, bool sink,
+    float out_scale, int part_keys, float* __restrict__ ws_acc, float* __restrict__ ws_ml, int row_base, int ws_rows) {
+  constexpr int kLd = KLd<KS>::v;
+  constexpr int kKF = (KS * 4 + kFT - 1) / kFT, kVF = (NV * 2 + kFT - 1) / kFT;  // 16-byte chunks per thread and tile
+  __shared__ __attribute__((aligned(16))) unsigned short kt[kKeys * kLd];     // [key][dim]
+  __shared__ __attribute__((aligned(16))) unsigned short vt[NV * 16 * kVLd];  // [value dim][permuted key]
+  int s, tok0;
+  if (!find_tile_rows(seq_cu, seq0, seq1, tq, blockIdx.x, s, tok0)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int group = heads / kv_heads;
+  const int kvh = blockIdx.y / hchunks, h0 = (blockIdx.y % hchunks) * hc;
+  const int nh = min(hc, group - h0);
+  const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0, ctx = seq_ctx[s];
+  const int ntok = min(tq, n - tok0);
+  const int p_first = ctx - n + tok0, p_last = p_first + ntok - 1;
+  const int lo_all = window > 0 ? max(0, p_first - window + 1) : 0;
+  const int lo = lo_all + blockIdx.z * part_keys;
+  const int hi = gridDim.z > 1 ? min(p_last, lo + part_keys - 1) : p_last;
+  const long Dc = (long)kv_heads * (dim + vdim);
+  const long koff = (long)kvh * dim, voff = (long)kv_heads * dim + (long)kvh * vdim;
+  const bool first_part = blockIdx.z == 0;
+  const float scale2 = scale * 1.44269504088896341f;
+  // this lane's rows: row sr = token sr / hc, head sr % hc of the group
+  bool sact[MT];
+  int head[MT], spos[MT], s_lo[MT];
+  long trow[MT];
+  bf16x8 qf[MT][KS];   // Q operands of the rows: dims 32 ks + 8 g .. + 7
+  f32x4 acc[MT][NV];
+  float m_run[MT], l_run[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int sr = 16 * (wave * MT + mt) + c;
+    const int srt = sr / hc, srh = sr % hc;
+    sact[mt] = srt < ntok && srh < nh;
+    head[mt] = kvh * group + h0 + (sact[mt] ? srh : 0);
+    trow[mt] = r0 + tok0 + (sact[mt] ? srt : 0);
+    spos[mt] = p_first + srt;
+    s_lo[mt] = window > 0 ? max(0, spos[mt] - window + 1) : 0;
+    const unsigned short* src = proj + trow[mt] * proj_ld + (long)head[mt] * dim;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = 32 * ks + 8 * g + e;
+        if (sact[mt] && d < dim) v[e] = src[d];
+      }
+      qf[mt][ks] = __builtin_bit_cast(bf16x8, v);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run[mt] = (sink && first_part) ? 0.f : -INFINITY;
+    l_run[mt] = (sink && first_part) ? 1.f : 0.f;
+  }
+  // tile fill: kFT threads per key; key 16 a + 4 gg + b of the tile sits in column 8 gg + 4 a + b of the value tile
+  const int fkey = tid / kFT, fk = tid % kFT;
+  const int vcol = 8 * ((fkey >> 2) & 3) + 4 * (fkey >> 4) + (fkey & 3);
+  const int kchunks = dim / 8, vchunks = vdim / 8;
+  u16x8 kf[kKF], vf[kVF];
+  auto fetch = [&](int j0) {
+    const int j = j0 + fkey;
+    const bool in = j <= hi;
+    const long kr = in ? ((long)seq_bt[(long)s * bt_width + j / block_size] * block_size + j % block_size) * Dc : 0;
+#pragma unroll
+    for (int i = 0; i < kKF; ++i) {
+      const int ch = fk + kFT * i;
+      kf[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (in && ch < kchunks) kf[i] = *reinterpret_cast<const u16x8*>(cache + kr + koff + 8 * ch);
+    }
+#pragma unroll
+    for (int i = 0; i < kVF; ++i) {
+      const int ch = fk + kFT * i;
+      vf[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (in && ch < vchunks) vf[i] = *reinterpret_cast<const u16x8*>(cache + kr + voff + 8 * ch);
+    }
+  };
+  if (lo <= hi) fetch(lo);
+  for (int j0 = lo; j0 <= hi; j0 += kKeys) {
+    __syncthreads();  // the previous tile's reads are done
+#pragma unroll
+    for (int i = 0; i < kKF; ++i) {
+      const int ch = fk + kFT * i;
+      if (ch < KS * 4) *reinterpret_cast<u16x8*>(kt + fkey * kLd + 8 * ch) = kf[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kVF; ++i) {
+      const int ch = fk + kFT * i;
+      if (ch < NV * 2) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vt[(8 * ch + e) * kVLd + (vcol ^ ((ch & 3) << 3))] = vf[i][e];
+      }
+    }
+    __syncthreads();
+    if (j0 + kKeys <= hi) fetch(j0 + kKeys);  // the next tile's loads fly during this tile's math
+    // S^T tiles: a = keys (16 per tile), b = 16 rows
+    f32x4 sc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) sc[mt][0] = sc[mt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(kt + (16 * nt + c) * kLd + 32 * ks + 8 * g));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          sc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[mt][ks], sc[mt][nt], 0, 0, 0);
+      }
+    }
+    bf16x8 pb8[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      // scores in the log2 domain (scale2 = scale * log2 e). A tile that every row of the wave sees whole
+      // (most tiles of a long window) skips the per-key visibility tests.
+      float v[8];
+      float mx = -INFINITY;
+      const bool whole = sact[mt] && j0 >= s_lo[mt] && j0 + kKeys - 1 <= min(spos[mt], hi);
+      if (__all(whole)) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          v[e] = sc[mt][e >> 2][e & 3] * scale2;
+          mx = fmaxf(mx, v[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int j = j0 + 16 * (e >> 2) + 4 * g + (e & 3);
+          const bool vis = sact[mt] && j <= hi && j <= spos[mt] && j >= s_lo[mt];
+          v[e] = vis ? sc[mt][e >> 2][e & 3] * scale2 : -INFINITY;
+          mx = fmaxf(mx, v[e]);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m_run[mt], mx);
+      float sum = 0.f;
+      u16x8 pk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(v[e] - mn);  // -inf - mn: 0 (mn is finite whenever a key is seen)
+        const unsigned short pb = f32_to_bf16(mn > -INFINITY ? p : 0.f);  // rounded to bf16: what is multiplied
+        pk[e] = pb;
+        sum += bf16_to_f32(pb);  // the sum of the weights that are actually multiplied
+      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      const float al = (mn > -INFINITY) ? __builtin_amdgcn_exp2f(m_run[mt] - mn) : 1.f;  // m_run = -inf: 0
+      l_run[mt] = l_run[mt] * al + sum;
+      m_run[mt] = mn;
+      if (__any(al != 1.f)) {  // the running maxima settle after a few tiles: most tiles skip this
+#pragma unroll
+        for (int j = 0; j < NV; ++j) acc[mt][j] *= al;
+      }
+      pb8[mt] = __builtin_bit_cast(bf16x8, pk);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const bf16x8 a = __builtin_bit_cast(
+          bf16x8, *reinterpret_cast<const u16x8*>(vt + (16 * j + c) * kVLd + 8 * (g ^ ((2 * j + (c >> 3)) & 3))));
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb8[mt], acc[mt][j], 0, 0, 0);
+    }
+  }
+  // lane (c, g) holds value dims 16 j + 4 g .. + 3 of its rows
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (!sact[mt]) continue;
+    if (gridDim.z > 1) {
+      const long wrow = ((long)blockIdx.z * heads + head[mt]) * ws_rows + (trow[mt] - row_base);
+      if (g == 0) { ws_ml[2 * wrow] = m_run[mt]; ws_ml[2 * wrow + 1] = l_run[mt]; }
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int d = 16 * j + 4 * g;
+        if (d < vdim) *reinterpret_cast<f32x4*>(ws_acc + wrow * vdim + d) = acc[mt][j];
+      }
+      continue;
+    }
+    float f = out_scale;
+    if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[trow[mt] * proj_ld + gate_off + head[mt]]));
+    f = l_run[mt] > 0.f ? f / l_run[mt] : 0.f;
+    unsigned short* dst = out + trow[mt] * out_ld + (long)head[mt] * vdim;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int d = 16 * j + 4 * g;
+      if (d >= vdim) continue;  // vdim % 8 == 0: the four dims are inside together
+      u16x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(acc[mt][j][e] * f);
+      *reinterpret_cast<u16x4*>(dst + d) = o;
+    }
+  }
+}
+
+// out[row_base + r, head] = sum_p acc_p e^(m_p - M) / sum_p l_p e^(m_p - M) * sigmoid(gate) * out_scale
+constexpr int kMaxRuns = 64;
+__global__ __launch_bounds__(128) void window_attention_reduce_kernel(
+    unsigned short* __restrict__ out, long out_ld, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
+    const unsigned short* __restrict__ proj, long proj_ld, int gate_off, int nparts, int heads, int ws_rows,
+    int row_base, int vdim, float out_scale) {
+  __shared__ float sc[kMaxRuns];  // each run's weight e^(m_p - M) / L * gate * scale, 0 for empty runs
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  if (tid < 64) {  // one wave: run p on lane p
+    const long w = ((long)min(tid, nparts - 1) * heads + h) * ws_rows + r;
+    const float m = tid < nparts ? ws_ml[2 * w] : -INFINITY;
+    const float l = tid < nparts ? ws_ml[2 * w + 1] : 0.f;
+    const float M = wave_max(m);
+    const float e = m > -INFINITY ? __builtin_amdgcn_exp2f(m - M) : 0.f;  // the runs' maxima are in the log2 domain
+    const float L = wave_sum(l * e);
+    float f = out_scale;
+    if (gate_off >= 0) f *= sigmoid_f(bf16_to_f32(proj[(long)(row_base + r) * proj_ld + gate_off + h]));
+    sc[tid] = L > 0.f ? e * f / L : 0.f;
+  }
+  __syncthreads();
+  const long trow = row_base + r;
+  for (int d = tid; d < vdim; d += 128) {
+    float o = 0.f;
+    for (int p = 0; p < nparts; ++p) o += ws_acc[(((long)p * heads + h) * ws_rows + r) * vdim + d] * sc[p];
+    out[trow * out_ld + (long)h * vdim + d] = f32_to_bf16(o);
+  }
+}
+
+template <int KS, int NV, int MT>
+void launch_mfma(unsigned short* out, long out_ld, const unsigned short* proj, long proj_ld, const unsigned short* cache,
+                 int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt, int bt_width, int seq0,
+                 int seq1, int rows_bound, int heads, int kv_heads, int dim, int vdim, int gate_off, float scale,
+                 int window, bool sink, float out_scale, int nparts, int part_keys, float* ws_acc, float* ws_ml,
+                 int row_base, hipStream_t s) {
+  const int group = heads / kv_heads;
+  const int rows = kRows * MT;
+  const int hc = min(group, rows);
+  const int hchunks = (group + hc - 1) / hc;
+  // split rows (decode): one token per workgroup; else as many consecutive tokens as fit the rows
+  const int tq = nparts > 1 ? 1 : rows / hc;
+  dim3 grid(rows_bound / tq + (seq1 - seq0), kv_heads * hchunks, nparts);
+  window_attention_mfma_kernel<KS, NV, MT><<<grid, kThreads, 0, s>>>(
+      out, out_ld, proj, proj_ld, cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1, tq, hc, hchunks,
+      heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, part_keys, ws_acc, ws_ml, row_base,
+      rows_bound);
+  if (nparts > 1)
+    window_attention_reduce_kernel<<<dim3(rows_bound, heads), 128, 0, s>>>(out, out_ld, ws_acc, ws_ml, proj, proj_ld,
+                                                                         gate_off, nparts, heads, rows_bound, row_base,
+                                                                         vdim, out_scale);
+}
+
+}  // namespace
+
+bool window_attention_mfma_ok(int dim, int vdim, long out_ld, long out_off) {
+  return dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 256 && out_ld % 4 == 0 && out_off % 4 == 0;
+}
+
+void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long proj_ld, const void* cache,
+                                  int block_size, const int* seq_cu, const int* seq_ctx, const int* seq_bt,
+                                  int bt_width, int seq0, int seq1, int rows_bound, int heads, int kv_heads, int dim,
+                                  int vdim, int gate_off, float scale, int window, bool sink, float out_scale,
+                                  int nparts, int part_keys, float* ws_acc, float* ws_ml, int row_base,
+                                  hipStream_t s) {
+  if (seq1 <= seq0 || rows_bound <= 0) return;
+#define HS_WA(KS, NV, MT)                                                                                           \
+  launch_mfma<KS, NV, MT>((unsigned short*)out, out_ld, (const unsigned short*)proj, proj_ld,                        \
+                          (const unsigned short*)cache, block_size, seq_cu, seq_ctx, seq_bt, bt_width, seq0, seq1,    \
+                          rows_bound, heads, kv_heads, dim, vdim, gate_off, scale, window, sink, out_scale, nparts,   \
+                          part_keys, ws_acc, ws_ml, row_base, s)
+  // two row tiles per wave where a prompt portion brings enough rows and the accumulators fit the registers
+  const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
+  const bool wide = nparts == 1 && (long)rows_bound * (heads / kv_heads) >= 128 * (long)(seq1 - seq0);
+  if (ks <= 2 && nv <= 4) { if (wide) HS_WA(2, 4, 2); else HS_WA(2, 4, 1); }
+  else if (ks <= 4 && nv <= 8) { if (wide) HS_WA(4, 8, 2); else HS_WA(4, 8, 1); }
+  else HS_WA(8, 16, 1);
+#undef HS_WA
+}
+
+}  // namespace hipserve

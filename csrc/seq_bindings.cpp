@@ -37,7 +37,7 @@ void scaled_add_group_rmsnorm(at::Tensor& out, at::Tensor& residual, const at::T
   TORCH_CHECK(groups >= 1 && H % groups == 0 && w.numel() == H && H + groups <= 15000, "group norm shape");
   if (mix.has_value()) {
     TORCH_CHECK(mix->scalar_type() == out.scalar_type() && mix->is_contiguous() && mix->sizes() == residual.sizes());
-    TORCH_CHECK(ls1.has_value() && ls1->scalar_type() == at::kFloat && ls1->numel() == H);
+    TORCH_CHECK(!ls1.has_value() || (ls1->scalar_type() == at::kFloat && ls1->is_contiguous() && ls1->numel() == H));
   }
   if (y.has_value()) {
     TORCH_CHECK(y->scalar_type() == out.scalar_type() && y->is_contiguous() && y->dim() == 2 && y->size(1) == H);

@@ -38,11 +38,16 @@ HIP_FLAGS = [
 ]
 
 # kernel libraries: name -> (shared object, kernel sources, host bindings). "core" is every
-# dense-transformer / sampling / quantisation kernel; "seq" the layer-list decoders' kernels
-# (plus the expert alignment of moe.hip), so a model of those designs builds only what it runs.
+# dense-transformer / sampling / quantisation kernel; "seq" the latent-attention / minGRU / table-MoE
+# kernels of the layer-list decoders (plus the expert alignment of moe.hip); "delta" their window
+# attention, delta-rule recurrences and activations. The residual + norm kernel is linked into both
+# of the latter, so a model of those designs builds only what it runs.
 LIBS = {
     "core": ("_C.so", ["kernels/*.hip"], "torch_bindings.cpp"),
-    "seq": ("_C_seq.so", ["kernels/seq/*.hip", "kernels/moe.hip"], "seq_bindings.cpp"),
+    "seq": ("_C_seq.so", ["kernels/seq/group_norm.hip", "kernels/seq/latent_attention*.hip", "kernels/seq/mingru.hip",
+                          "kernels/seq/expert_ffn.hip", "kernels/moe.hip"], "seq_bindings.cpp"),
+    "delta": ("_C_delta.so", ["kernels/seq/group_norm.hip", "kernels/seq/window_attention*.hip",
+                              "kernels/seq/delta_scan.hip"], "seq_delta_bindings.cpp"),
 }
 
 
@@ -95,7 +100,7 @@ def _compile(src, obj, cmd, want):
 
 def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = False, lib: str = "core") -> str:
     """Build one kernel library of ``LIBS`` (gfx950 kernels + torch op registrations):
-    ``core`` = hipserve/_C.so, ``seq`` = hipserve/_C_seq.so."""
+    ``core`` = hipserve/_C.so, ``seq`` = hipserve/_C_seq.so, ``delta`` = hipserve/_C_delta.so."""
     if not os.path.exists(HIPCC):
         raise RuntimeError(f"hipcc not found at {HIPCC}")
     so_name, patterns, bindings = LIBS[lib]
@@ -218,6 +223,7 @@ def build_all(force: bool = False, jobs: int | None = None, verbose: bool = True
     rt = build_runtime(force=force, verbose=verbose)
     so = build_kernels(force=force, jobs=jobs, verbose=verbose)
     build_kernels(force=force, jobs=jobs, verbose=verbose, lib="seq")
+    build_kernels(force=force, jobs=jobs, verbose=verbose, lib="delta")
     return so, rt
 
 

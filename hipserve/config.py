@@ -602,9 +602,113 @@ class TableMoESpec:
 
 
 @dataclass(frozen=True)
+class WindowAttentionSpec:
+    """Grouped-query attention over a sliding window (``window`` keys: the token itself and
+    the ``window - 1`` before it; 0 = plain causal) with rotate-half rotary positions on the
+    first ``rot_dims`` dims of every head. Options, each independent of the others:
+    ``sink`` adds one to the softmax denominator (a key of score 0 without a value),
+    ``gate`` multiplies head h's output by sigmoid of a per-head projection of the mixer input,
+    ``bias`` adds biases in the q / k / v projections, ``qk_norm`` applies a weighted RMS norm
+    over the WHOLE q (and k) projection before the rotation, ``v_norm`` divides every value
+    head by its root mean square (cached so)."""
+    heads: int
+    kv_heads: int
+    dim: int            # query / key dims per head
+    vdim: int           # value dims per head
+    scale: float
+    window: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    sink: bool = False
+    gate: bool = False
+    bias: bool = False
+    qk_norm: bool = False
+    v_norm: bool = False
+
+    kind = "attention"
+
+    @property
+    def q_size(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def k_size(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def v_size(self) -> int:
+        return self.kv_heads * self.vdim
+
+    @property
+    def cache_dim(self) -> int:
+        """Cached elements per token: all key heads, then all value heads."""
+        return self.k_size + self.v_size
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """Gated delta rule: per head a ``dim x vdim`` state that decays by one number per token
+    and is corrected towards the token's value along its unit key; q, k and v pass a causal
+    convolution of ``conv`` taps and SiLU first. ``kv_heads`` query / key heads serve ``heads``
+    value heads."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+
+    kind = "delta"
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    @property
+    def proj_size(self) -> int:
+        """Merged input projection: q | k | v | beta | decay | output gate."""
+        return self.conv_channels + 2 * self.heads + self.heads * self.vdim
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """Generalized delta rule: per head a ``dim x dim`` state with a decay and a removal rate
+    per key channel; the decay comes from a ``decay_rank`` bottleneck."""
+    heads: int
+    dim: int
+    decay_rank: int = 0     # read from the checkpoint when 0
+
+    kind = "delta_rule"
+
+    @property
+    def size(self) -> int:
+        return self.heads * self.dim
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers on the same input, their outputs summed with fixed weights."""
+    left: object
+    right: object
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+
+    kind = "parallel"
+
+
+@dataclass(frozen=True)
+class DenseFFSpec:
+    """down(act(up(x))) with one of the op set's elementwise activations."""
+    ff: int
+    act: str = "xielu"
+
+    kind = "dense"
+
+
+@dataclass(frozen=True)
 class HybridLayerSpec:
-    mixer: object               # LatentAttentionSpec | MinGRUSpec
-    mlp: object | None          # TableMoESpec | None
+    mixer: object               # a mixer spec of this section
+    mlp: object | None          # TableMoESpec | DenseFFSpec | None
+    weights_of: int | None = None   # the layer whose weights this one uses (its own when None)
 
 
 @dataclass(frozen=True)
@@ -696,11 +800,113 @@ class HybridConfig:
             logit_scale=float(d.get("logit_scale", 1.0)), bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
 
 
+@dataclass(frozen=True)
+class FikizenConfig:
+    """Fikizen: a pre-norm decoder given as a list of layers, each with one mixer (windowed
+    sink attention with an output gate, a gated delta rule, or attention and a generalized
+    delta rule in parallel) and an optional dense feed-forward. A layer can use another
+    layer's weights (``weights_of``) with a cache / state of its own. Logits are soft-capped."""
+    name: str = "fikizen"
+    architecture: str = "fikizen"
+    family: str = "fikizen"
+    hidden_size: int = 256
+    vocab_size: int = 512
+    layers: tuple = ()
+    norm_eps: float = 1e-6
+    logit_softcap: float = 0.0
+    max_position_embeddings: int = 1 << 20   # rotary angles are computed, not tabulated
+    default_model_len: int = 32768
+    bos_token_id: int | None = None
+    eos_token_id: tuple = ()
+    vision: object = None
+    num_experts: int = 0
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list:
+        """Layer runs in execution order: (index of the layer that holds the weights, 0, False)."""
+        return [(i if l.weights_of is None else l.weights_of, 0, False) for i, l in enumerate(self.layers)]
+
+    def num_params(self) -> int:
+        H, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+
+        def mixer(m):
+            if isinstance(m, WindowAttentionSpec):
+                return H * (m.q_size + m.cache_dim + (m.heads if m.gate else 0)) + m.heads * m.vdim * H
+            if isinstance(m, GatedDeltaSpec):
+                return H * m.proj_size + m.heads * m.vdim * H
+            if isinstance(m, DeltaRuleSpec):
+                return 6 * H * m.size
+            return mixer(m.left) + mixer(m.right)
+
+        for l in self.layers:
+            if l.weights_of is None:
+                n += mixer(l.mixer) + (2 * l.mlp.ff * H if l.mlp is not None else 0)
+        return n
+
+    def replace(self, **kw) -> "FikizenConfig":
+        return dataclasses.replace(self, **kw)
+
+    @staticmethod
+    def attention_spec(m: dict, **flags) -> WindowAttentionSpec:
+        rot = m.get("rot") or {}
+        return WindowAttentionSpec(
+            heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+            scale=float(m["scale"]), window=int((m.get("mask") or {}).get("size") or 0),
+            rot_dims=int(rot.get("dims") or 0), rot_base=float(rot.get("base", 10000.0)), sink=True, **flags)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "model") -> "FikizenConfig":
+        layers = []
+        for l in d["layers"]:
+            m, kind = l["mixer"], l["type"]
+            if kind == "attention":
+                mixer = FikizenConfig.attention_spec(m, gate=True)
+            elif kind == "delta":
+                mixer = GatedDeltaSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                       vdim=int(m["vdim"]), conv=int(m["conv"]))
+            elif kind == "parallel":
+                mixer = ParallelMixerSpec(
+                    left=FikizenConfig.attention_spec(m["left"], bias=True, qk_norm=True, v_norm=True),
+                    right=DeltaRuleSpec(heads=int(m["right"]["heads"]), dim=int(m["right"]["dim"]),
+                                        decay_rank=int(m["right"].get("decay_rank") or 0)),
+                    left_scale=float(m.get("left_scale", 1.0)), right_scale=float(m.get("right_scale", 1.0)))
+            else:
+                raise NotImplementedError(f"unknown mixer {kind!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") != "dense":
+                    raise NotImplementedError(f"unknown feed-forward {f.get('kind')!r}")
+                mlp = DenseFFSpec(ff=int(f["ff"]))
+            wo = l.get("weights_of")
+            layers.append(HybridLayerSpec(mixer, mlp, None if wo is None else int(wo)))
+        for i, l in enumerate(layers):
+            if l.weights_of is not None:
+                j = l.weights_of
+                if not (0 <= j < len(layers)) or layers[j].weights_of is not None:
+                    raise ValueError(f"layer {i}: weights_of must name a layer with weights of its own")
+                if (layers[j].mixer, layers[j].mlp) != (l.mixer, l.mlp):
+                    raise ValueError(f"layer {i} differs from layer {j}, whose weights it uses")
+        norm = d.get("norm") or {}
+        eos = d.get("eos_token_id", ())
+        eos = tuple(eos) if isinstance(eos, (list, tuple)) else (eos,)
+        return FikizenConfig(
+            name=name, hidden_size=int(d["width"]), vocab_size=int(d["vocab"]), layers=tuple(layers),
+            norm_eps=float(norm.get("eps", 1e-6)), logit_softcap=float(d.get("logit_softcap") or 0.0),
+            bos_token_id=d.get("bos_token_id"), eos_token_id=eos)
+
+
 def config_from_dict(d: dict, name: str = "model"):
     """Model config of a ``config.json``: the layer-list designs are recognised by their
     ``architecture`` key, everything else is a HuggingFace config."""
-    if str(d.get("architecture", "")).lower() == "kesirax":
+    arch = str(d.get("architecture", "")).lower()
+    if arch == "kesirax":
         return HybridConfig.from_dict(d, name=name)
+    if arch == "fikizen":
+        return FikizenConfig.from_dict(d, name=name)
     return ModelConfig.from_hf_dict(d, name=name)
 
 
@@ -725,4 +931,35 @@ PRESETS.update({
                                    dict(heads=8, dim=64, rot_dim=32, vdim=64, q_rank=192, kv_rank=128,
                                         scale=96 ** -0.5, window=160, rot_base=50000.0),
                                    768, dict(experts=8, top=2, ff=256), "agag", loop=(0, 2, 2), groups=2),
+})
+
+
+def _mini_fikizen(name, H, V, attn, left, delta, rule, ff, order, scales=(0.75, 1.25), softcap=20.0):
+    """order: 'd' gated delta rule (no feed-forward), 'a' gated sink attention + feed-forward, 'p' parallel
+    mixer + feed-forward, 'A' the first 'a' layer's weights once more."""
+    a = WindowAttentionSpec(sink=True, gate=True, **attn)
+    p = ParallelMixerSpec(WindowAttentionSpec(sink=True, bias=True, qk_norm=True, v_norm=True, **left),
+                          DeltaRuleSpec(**rule), *scales)
+    f = DenseFFSpec(ff)
+    first = order.index("a") if "A" in order else None
+    spec = {"d": HybridLayerSpec(GatedDeltaSpec(**delta), None), "a": HybridLayerSpec(a, f),
+            "p": HybridLayerSpec(p, f), "A": HybridLayerSpec(a, f, first)}
+    return FikizenConfig(name=name, hidden_size=H, vocab_size=V, layers=tuple(spec[c] for c in order),
+                         logit_softcap=softcap, eos_token_id=(2,), bos_token_id=1)
+
+
+PRESETS.update({
+    # CPU plumbing size
+    "tiny-fikizen": _mini_fikizen("tiny-fikizen", 64, 320,
+                                  dict(heads=4, kv_heads=2, dim=16, vdim=24, scale=0.25, window=24, rot_dims=8),
+                                  dict(heads=3, kv_heads=3, dim=16, vdim=16, scale=0.25, window=16, rot_dims=16),
+                                  dict(heads=4, kv_heads=2, dim=8, vdim=12, conv=3), dict(heads=2, dim=16, decay_rank=8),
+                                  96, "apdAd"),
+    # GPU-test size
+    "small-fikizen": _mini_fikizen("small-fikizen", 512, 1024,
+                                   dict(heads=8, kv_heads=2, dim=64, vdim=64, scale=0.125, window=160, rot_dims=32,
+                                        rot_base=5e5),
+                                   dict(heads=8, kv_heads=4, dim=64, vdim=64, scale=0.125, window=80, rot_dims=64),
+                                   dict(heads=8, kv_heads=4, dim=64, vdim=64, conv=3), dict(heads=8, dim=64, decay_rank=32),
+                                   1536, "adAp"),
 })

@@ -19,13 +19,30 @@ them is one op of the op set:
 * table MoE: expert ids looked up by token id -> ``moe_align`` tiles -> two
   ``expert_gemm`` launches (squared-ReLU in the first one's epilogue); the weighted
   combine is folded into the residual update (``scaled_add_group_rmsnorm``).
+* window attention: merged [q | k | v | gate] projection (biases in its epilogue) ->
+  ``attn_prepare`` (whole-projection q / k norm, rotation, value norm, paged cache write) ->
+  ``window_attention`` (sliding window, softmax with a sink, per-head output gate) ->
+  output projection.
+* gated delta rule: merged [q | k | v | beta | decay | gate] projection -> ``gated_delta``
+  (causal convolution + SiLU, unit q / k, the recurrence from the sequence's state slot,
+  per-head output norm and SiLU gate) -> output projection.
+* generalized delta rule: merged [r | k | v | a | g | decay bottleneck] projection -> tanh ->
+  decay up-projection (32-bit result) -> ``delta_rule`` (decay, removal rate, unit key, the
+  recurrence, per-head output norm and sigmoid gate) -> output projection.
+* parallel mixer: both halves write their scaled head outputs side by side into one
+  buffer, and ONE output projection over the concatenated weights sums them.
+* dense feed-forward: up projection -> ``activation`` -> down projection.
+
+A mixer's ``forward(h, meta, cache, state)`` gets the layer run's paged cache and state
+tensors (None where it has none); ``cache_dim`` / ``state_shapes`` say what a run needs.
 """
 from __future__ import annotations
 
 import torch
 import torch.nn.functional as F
 
-from ..config import LatentAttentionSpec, MinGRUSpec, TableMoESpec
+from ..config import (DeltaRuleSpec, DenseFFSpec, GatedDeltaSpec, LatentAttentionSpec, MinGRUSpec, ParallelMixerSpec,
+                      TableMoESpec, WindowAttentionSpec)
 
 MOE_TILE = 32        # slots per expert tile of the expert GEMMs ...
 MOE_TILE_LARGE = 64  # ... when every expert has several tiles' worth of rows on average
@@ -224,3 +241,258 @@ class TableMoE:
         y = torch.empty(cap, H, dtype=h.dtype, device=dev)
         op.prefill_gemm_packed_grouped(y, act, pd, H, 0, tile_expert, ntiles, gemm.PW_WM, gemm.PW_RW)
         return y, pair_slot
+
+
+def _linear32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x . w^T with a 32-bit result (inputs of the recurrences' decays stay 32-bit)."""
+    if x.dtype == torch.float32:
+        return F.linear(x, w)
+    if x.is_cuda:
+        return torch.mm(x, w.t(), out_dtype=torch.float32)
+    return F.linear(x.float(), w.float())
+
+
+def _rand(gen, *shape, std=1.0):
+    return torch.randn(*shape, generator=gen) * std
+
+
+class WindowAttention:
+    cache_dim = property(lambda self: self.spec.cache_dim)
+    state_shapes = None
+
+    def __init__(self, spec: WindowAttentionSpec, hidden: int, eps: float, device, dtype, ops):
+        self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
+        self.w_in = None     # [q | k | v | gate, hidden]
+        self.b_in = None     # [same] or None
+        self.q_norm = self.k_norm = None   # fp32 [heads * dim], [kv_heads * dim]
+        self.w_o = None      # [hidden, heads * vdim]
+        half = spec.rot_dims // 2
+        i = torch.arange(half, dtype=torch.float32)
+        # f_i = base^(-2i / dims), 32-bit
+        self.inv_freq = torch.pow(torch.tensor(spec.rot_base, dtype=torch.float32),
+                                  -2.0 * i / max(spec.rot_dims, 1)).to(device)
+        self.gate_off = spec.q_size + spec.cache_dim if spec.gate else -1
+
+    @property
+    def out_size(self) -> int:
+        return self.spec.heads * self.spec.vdim
+
+    def load(self, get, prefix: str):
+        s, dt, dev = self.spec, self.dtype, self.device
+        names = ["q", "k", "v"] + (["g"] if s.gate else [])
+        self.w_in = torch.cat([get(prefix + n) for n in names], 0).to(dev, dt).contiguous()
+        if s.bias:
+            b = [get(prefix + n + ".b") for n in ("q", "k", "v")] + ([torch.zeros(s.heads)] if s.gate else [])
+            self.b_in = torch.cat([x.float() for x in b]).to(dev, dt).contiguous()
+        if s.qk_norm:
+            self.q_norm = get(prefix + "q.norm").to(dev, torch.float32)
+            self.k_norm = get(prefix + "k.norm").to(dev, torch.float32)
+        self.w_o = get(prefix + "o").to(dev, dt).contiguous()
+
+    def init_random(self, gen, std: float):
+        s, H = self.spec, self.hidden
+        t = {"q": _rand(gen, s.q_size, H, std=std * 4), "k": _rand(gen, s.k_size, H, std=std * 4),
+             "v": _rand(gen, s.v_size, H, std=std * 4), "o": _rand(gen, H, self.out_size, std=std)}
+        if s.gate:
+            t["g"] = _rand(gen, s.heads, H, std=std * 4)
+        if s.bias:
+            t.update({"q.b": _rand(gen, s.q_size, std=0.3), "k.b": _rand(gen, s.k_size, std=0.3),
+                      "v.b": _rand(gen, s.v_size, std=0.3)})
+        if s.qk_norm:
+            t.update({"q.norm": 1.0 + 0.2 * _rand(gen, s.q_size), "k.norm": 1.0 + 0.2 * _rand(gen, s.k_size)})
+        return t
+
+    def mix(self, h, meta, cache, state, out, out_scale: float = 1.0):
+        """Head outputs (before the output projection), times ``out_scale``, into ``out`` [T, heads * vdim]
+        (a column slice of a wider buffer is fine)."""
+        s, ops = self.spec, self.ops
+        proj = F.linear(h, self.w_in, self.b_in)
+        ops.attn_prepare(proj, cache, meta, self.inv_freq, s, self.q_norm, self.k_norm, self.eps)
+        ops.window_attention(out, proj, cache, meta, s, self.gate_off, out_scale)
+        return out
+
+    def forward(self, h, meta, cache, state):
+        out = torch.empty(h.shape[0], self.out_size, device=h.device, dtype=h.dtype)
+        return F.linear(self.mix(h, meta, cache, state, out), self.w_o)
+
+
+class GatedDelta:
+    cache_dim = 0
+
+    def __init__(self, spec: GatedDeltaSpec, hidden: int, eps: float, device, dtype, ops):
+        self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
+        self.w_in = None      # [q | k | v | beta | decay | gate, hidden]
+        self.conv_w = None    # fp32 [conv channels, taps]
+        self.a_log = self.dt_bias = None  # fp32 [heads]
+        self.norm = None      # fp32 [vdim]
+        self.w_o = None
+
+    @property
+    def out_size(self) -> int:
+        return self.spec.heads * self.spec.vdim
+
+    def state_shapes(self, slots: int):
+        s = self.spec
+        return [(slots, s.heads, s.dim, s.vdim), (slots, max(s.conv - 1, 1), s.conv_channels)]
+
+    def load(self, get, prefix: str):
+        dt, dev = self.dtype, self.device
+        self.w_in = torch.cat([get(prefix + n) for n in ("q", "k", "v", "b", "a", "g")], 0).to(dev, dt).contiguous()
+        self.conv_w = torch.cat([get(prefix + n + ".conv") for n in ("q", "k", "v")], 0).to(dev, torch.float32).contiguous()
+        self.a_log = get(prefix + "A_log").to(dev, torch.float32)
+        self.dt_bias = get(prefix + "dt_bias").to(dev, torch.float32)
+        self.norm = get(prefix + "norm").to(dev, torch.float32)
+        self.w_o = get(prefix + "o").to(dev, dt).contiguous()
+
+    def init_random(self, gen, std: float):
+        s, H = self.spec, self.hidden
+        qk = s.kv_heads * s.dim
+        t = {"q": _rand(gen, qk, H, std=std * 4), "k": _rand(gen, qk, H, std=std * 4),
+             "v": _rand(gen, self.out_size, H, std=std * 4), "b": _rand(gen, s.heads, H, std=std * 4),
+             "a": _rand(gen, s.heads, H, std=std * 4), "g": _rand(gen, self.out_size, H, std=std * 4),
+             "A_log": _rand(gen, s.heads, std=0.5) - 1.0, "dt_bias": _rand(gen, s.heads, std=0.5),
+             "norm": 1.0 + 0.2 * _rand(gen, s.vdim), "o": _rand(gen, H, self.out_size, std=std)}
+        for n, c in (("q", qk), ("k", qk), ("v", self.out_size)):
+            t[n + ".conv"] = _rand(gen, c, s.conv, std=0.5)
+        return t
+
+    def mix(self, h, meta, cache, state, out, out_scale: float = 1.0):
+        assert out_scale == 1.0
+        proj = F.linear(h, self.w_in)
+        self.ops.gated_delta(out, state, proj, self.conv_w, self.a_log, self.dt_bias, self.norm, self.spec, self.eps, meta)
+        return out
+
+    def forward(self, h, meta, cache, state):
+        out = torch.empty(h.shape[0], self.out_size, device=h.device, dtype=h.dtype)
+        return F.linear(self.mix(h, meta, cache, state, out), self.w_o)
+
+
+class DeltaRule:
+    cache_dim = 0
+
+    def __init__(self, spec: DeltaRuleSpec, hidden: int, eps: float, device, dtype, ops):
+        self.spec, self.hidden, self.eps, self.device, self.dtype, self.ops = spec, hidden, eps, device, dtype, ops
+        self.w_in = None    # [r | k | v | a | g | decay bottleneck, hidden]
+        self.w2 = None      # [heads * dim, rank]
+        self.a_b = self.w0 = self.norm = None   # fp32 [heads * dim]
+        self.w_o = None
+
+    @property
+    def out_size(self) -> int:
+        return self.spec.size
+
+    def state_shapes(self, slots: int):
+        s = self.spec
+        return [(slots, s.heads, s.dim, s.dim)]
+
+    def load(self, get, prefix: str):
+        dt, dev = self.dtype, self.device
+        self.w_in = torch.cat([get(prefix + n) for n in ("r", "k", "v", "a", "g", "w1")], 0).to(dev, dt).contiguous()
+        self.w2 = get(prefix + "w2").to(dev, dt).contiguous()
+        self.a_b = get(prefix + "a.b").to(dev, torch.float32)
+        self.w0 = get(prefix + "w0").to(dev, torch.float32)
+        self.norm = get(prefix + "norm").to(dev, torch.float32)
+        self.w_o = get(prefix + "o").to(dev, dt).contiguous()
+
+    def init_random(self, gen, std: float):
+        s, H, N = self.spec, self.hidden, self.spec.size
+        rank = s.decay_rank or max(8, N // 8)
+        t = {n: _rand(gen, N, H, std=std * 4) for n in ("r", "k", "v", "a", "g")}
+        t.update({"w1": _rand(gen, rank, H, std=std * 4), "w2": _rand(gen, N, rank, std=0.5), "w0": _rand(gen, N),
+                  "a.b": _rand(gen, N, std=0.5), "norm": 1.0 + 0.2 * _rand(gen, N), "o": _rand(gen, H, N, std=std)})
+        return t
+
+    def mix(self, h, meta, cache, state, out, out_scale: float = 1.0):
+        N, ops = self.spec.size, self.ops
+        proj = F.linear(h, self.w_in)
+        low = torch.empty(h.shape[0], self.w2.shape[1], device=h.device, dtype=h.dtype)
+        ops.activation(low, proj[:, 5 * N:], "tanh")
+        wl = _linear32(low, self.w2)
+        ops.delta_rule(out, state, proj, wl, self.a_b, self.w0, self.norm, self.spec, self.eps, meta, out_scale)
+        return out
+
+    def forward(self, h, meta, cache, state):
+        out = torch.empty(h.shape[0], self.out_size, device=h.device, dtype=h.dtype)
+        return F.linear(self.mix(h, meta, cache, state, out), self.w_o)
+
+
+class ParallelMixer:
+    """left_scale * left(h) + right_scale * right(h): both halves write their scaled head outputs
+    into one [T, left | right] buffer; one GEMM with the concatenated output weights sums them."""
+
+    def __init__(self, spec: ParallelMixerSpec, hidden: int, eps: float, device, dtype, ops):
+        self.spec, self.hidden, self.device, self.dtype, self.ops = spec, hidden, device, dtype, ops
+        self.left = make_mixer(spec.left, hidden, eps, device, dtype, ops)
+        self.right = make_mixer(spec.right, hidden, eps, device, dtype, ops)
+        self.w_o = None      # [hidden, left out | right out]
+
+    @property
+    def cache_dim(self) -> int:
+        assert not (self.left.cache_dim and self.right.cache_dim), "one paged cache per layer run"
+        return self.left.cache_dim or self.right.cache_dim
+
+    def state_shapes(self, slots: int):
+        assert not (self.left.state_shapes and self.right.state_shapes), "one state per layer run"
+        f = self.left.state_shapes or self.right.state_shapes
+        return f(slots) if f else []
+
+    def load(self, get, prefix: str):
+        self.left.load(get, prefix + "left.")
+        self.right.load(get, prefix + "right.")
+        self.w_o = torch.cat([self.left.w_o, self.right.w_o], 1).contiguous()
+        self.left.w_o = self.right.w_o = None
+
+    def init_random(self, gen, std: float):
+        t = {"left." + k: v for k, v in self.left.init_random(gen, std).items()}
+        t.update({"right." + k: v for k, v in self.right.init_random(gen, std).items()})
+        return t
+
+    def forward(self, h, meta, cache, state):
+        a, b = self.left.out_size, self.right.out_size
+        buf = torch.empty(h.shape[0], a + b, device=h.device, dtype=h.dtype)
+        self.left.mix(h, meta, cache, state, buf[:, :a], self.spec.left_scale)
+        self.right.mix(h, meta, cache, state, buf[:, a:], self.spec.right_scale)
+        return F.linear(buf, self.w_o)
+
+
+class DenseFF:
+    def __init__(self, spec: DenseFFSpec, hidden: int, device, dtype, ops):
+        self.spec, self.hidden, self.device, self.dtype, self.ops = spec, hidden, device, dtype, ops
+        self.w_up = self.w_down = None
+        self.c0 = self.c1 = 0.0     # xielu: softplus(p), 1/2 + softplus(q)
+
+    def load(self, get, prefix: str):
+        dt, dev = self.dtype, self.device
+        self.w_up = get(prefix + "up").to(dev, dt).contiguous()
+        self.w_down = get(prefix + "down").to(dev, dt).contiguous()
+        if self.spec.act == "xielu":
+            sp = F.softplus(get(prefix + "act").to(torch.float32))
+            self.c0, self.c1 = float(sp[0]), float(torch.tensor(0.5) + sp[1])
+
+    def init_random(self, gen, std: float):
+        t = {"up": _rand(gen, self.spec.ff, self.hidden, std=std * 4), "down": _rand(gen, self.hidden, self.spec.ff, std=std)}
+        if self.spec.act == "xielu":
+            t["act"] = _rand(gen, 2, std=0.5)
+        return t
+
+    def forward(self, h):
+        up = F.linear(h, self.w_up)
+        self.ops.activation(up, up, self.spec.act, self.c0, self.c1)
+        return F.linear(up, self.w_down)
+
+
+def make_mixer(spec, hidden: int, eps: float, device, dtype, ops):
+    """The weight holder of a mixer spec (the layer-list designs' common factory)."""
+    if isinstance(spec, WindowAttentionSpec):
+        return WindowAttention(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, GatedDeltaSpec):
+        return GatedDelta(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, DeltaRuleSpec):
+        return DeltaRule(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, ParallelMixerSpec):
+        return ParallelMixer(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, LatentAttentionSpec):
+        return LatentAttention(spec, hidden, eps, device, dtype, ops)
+    if isinstance(spec, MinGRUSpec):
+        return MinGRU(spec, hidden, eps, device, dtype, ops)
+    raise NotImplementedError(type(spec).__name__)

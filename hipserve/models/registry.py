@@ -21,6 +21,7 @@ ARCHITECTURES = {
     "llama": ("hipserve.models.llama", "LlamaModel", "hipserve.weights.safetensors_loader:load_hf_weights"),
     "mixtral": ("hipserve.models.llama", "LlamaModel", "hipserve.weights.safetensors_loader:load_hf_weights"),
     "kesirax": ("hipserve.models.kesirax", "KesiraxModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
+    "fikizen": ("hipserve.models.fikizen", "FikizenModel", "hipserve.weights.safetensors_loader:load_named_tensors"),
 }
 
 

@@ -1,8 +1,8 @@
 """hipserve op library.
 
 ``KernelOps`` calls the hand-written gfx950 kernels in ``hipserve/_C.so``
-(``torch.ops.hipserve.*``) and, for the layer-list decoders, ``hipserve/_C_seq.so``
-(``torch.ops.hipserve_seq.*``); each library is loaded at the first use of one of its kernels. ``ReferenceOps`` is the plain-PyTorch oracle used by
+(``torch.ops.hipserve.*``) and, for the layer-list decoders, ``hipserve/_C_seq.so`` and
+``hipserve/_C_delta.so`` (``torch.ops.hipserve_seq.*``, ``torch.ops.hipserve_delta.*``); each library is loaded at the first use of one of its kernels. ``ReferenceOps`` is the plain-PyTorch oracle used by
 the CPU plumbing engine and by the numerics tests. The choice is made ONCE, when
 an engine is built for a device — never per call. On a GPU device the native
 library is mandatory: a missing/unloadable ``_C.so`` raises instead of silently
@@ -20,9 +20,11 @@ from . import reference as ref
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 _LIB = os.path.join(_PKG, "_C.so")
 _LIB_SEQ = os.path.join(_PKG, "_C_seq.so")  # the layer-list decoders' kernels (torch.ops.hipserve_seq)
+_LIB_DELTA = os.path.join(_PKG, "_C_delta.so")  # ... window attention / delta rules (torch.ops.hipserve_delta)
 _lock = threading.Lock()
 _loaded = False
 _loaded_seq = False
+_loaded_delta = False
 
 
 def library_path() -> str:
@@ -63,6 +65,21 @@ def load_seq_library() -> str:
         return _LIB_SEQ
 
 
+def load_delta_library() -> str:
+    """Load hipserve/_C_delta.so into torch.ops (idempotent); built first when it is missing."""
+    global _loaded_delta
+    with _lock:
+        if _loaded_delta:
+            return _LIB_DELTA
+        if not os.path.exists(_LIB_DELTA):
+            from .._build import build_kernels
+
+            build_kernels(lib="delta")
+        torch.ops.load_library(_LIB_DELTA)
+        _loaded_delta = True
+        return _LIB_DELTA
+
+
 def native_available() -> bool:
     try:
         load_library()
@@ -79,6 +96,10 @@ class KernelOps:
     def __init__(self):
         self._core = None
         self._seq_ops = None
+        self._delta_ops = None
+        # the library whose copy of the shared residual + norm kernel runs ("seq" / "delta"): a model sets it
+        # to the one its mixers load anyway, so it never builds or loads the other
+        self.norm_library = "seq"
 
     @property
     def _op(self):
@@ -94,6 +115,13 @@ class KernelOps:
             load_seq_library()
             self._seq_ops = torch.ops.hipserve_seq
         return self._seq_ops
+
+    @property
+    def _delta(self):
+        if self._delta_ops is None:
+            load_delta_library()
+            self._delta_ops = torch.ops.hipserve_delta
+        return self._delta_ops
 
     def rmsnorm(self, out, x, w, eps, out8=None):
         """out8: (e4m3 [rows, hidden] uint8, scales fp32 [rows]) per-token FP8 copy of out."""
@@ -181,7 +209,8 @@ class KernelOps:
     # ---- layer-list decoders (csrc/kernels/seq/*.hip; bf16 or true fp32 activations)
     def scaled_add_group_rmsnorm(self, out, residual, w, groups, eps, mix=None, ls1=None, y=None, pair_slot=None,
                                  top=0, ls2=None, extra=None):
-        self._seq.scaled_add_group_rmsnorm(out, residual, w, groups, eps, mix, ls1, y, pair_slot, top, ls2, extra)
+        lib = self._delta if self.norm_library == "delta" else self._seq
+        lib.scaled_add_group_rmsnorm(out, residual, w, groups, eps, mix, ls1, y, pair_slot, top, ls2, extra)
         return out
 
     def latent_prepare(self, cq, cache, proj, positions, slots, q_norm, kv_norm, inv_freq, q_rank, kv_rank,
@@ -240,6 +269,66 @@ class KernelOps:
 
     def mingru_scan(self, y, state, proj, b_z, b_x, meta):
         self._seq.mingru_scan(y, state, proj, b_z, b_x, meta.seq_cu, meta.seq_ctx, meta.seq_state, meta.max_q)
+
+    def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
+        self._delta.attn_prepare(proj, cache, meta.positions, meta.slot_mapping, inv_freq, sp.heads, sp.kv_heads,
+                               sp.dim, sp.vdim, q_norm if sp.qk_norm else None, k_norm if sp.qk_norm else None,
+                               sp.v_norm, eps)
+
+    WINDOW_PREFILL_TQ = 4  # tokens per workgroup of a prompt portion (x the query heads of one key/value head)
+    # bf16 runs the MFMA kernel (HIPSERVE_WINDOW_MFMA=0: the generic kernel, as fp32 does)
+    WINDOW_MFMA = os.environ.get("HIPSERVE_WINDOW_MFMA", "1") != "0"
+    WINDOW_DECODE_RUN = 128  # keys per run of a decode row (a multiple of 32)
+
+    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0):
+        """Prompt portions (the step's first sequences) run several tokens per workgroup, decode
+        rows one token per workgroup."""
+        nseq = meta.seq_ctx.shape[0]
+        nd = meta.num_decode
+        npf, Tp = nseq - nd, meta.num_prefill_tokens
+        if (proj.dtype == torch.bfloat16 and self.WINDOW_MFMA
+                and self._delta.window_attention_mfma_ok(sp.dim, sp.vdim, out.stride(0), out.storage_offset())):
+            # bf16: the matrix-core kernel; decode rows split their keys into runs merged by a reduce kernel
+            args = (sp.heads, sp.kv_heads, sp.dim, sp.vdim, gate_off, sp.scale, sp.window, sp.sink, out_scale)
+            if npf:
+                self._delta.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, 0, npf, Tp,
+                                                *args, 1, 0, None, None, 0)
+            if nd:
+                span = min(sp.window, meta.max_ctx or sp.window) if sp.window > 0 else meta.max_ctx
+                part = self.WINDOW_DECODE_RUN
+                while -(-span // part) > 64:
+                    part *= 2
+                nparts = max(1, -(-span // part))
+                ws_acc = ws_ml = None
+                if nparts > 1:
+                    ws_acc = torch.empty(nparts, sp.heads, nd, sp.vdim, device=proj.device, dtype=torch.float32)
+                    ws_ml = torch.empty(nparts, sp.heads, nd, 2, device=proj.device, dtype=torch.float32)
+                self._delta.window_attention_mfma(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, npf, nseq, nd,
+                                                *args, nparts, part, ws_acc, ws_ml, Tp)
+            return
+        for s0, s1, rows, tq in ((0, npf, Tp, self.WINDOW_PREFILL_TQ), (npf, nseq, nd, 1)):
+            if s1 > s0:
+                self._delta.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, s0, s1, rows, tq,
+                                           sp.heads, sp.kv_heads, sp.dim, sp.vdim, gate_off, sp.scale, sp.window,
+                                           sp.sink, out_scale)
+
+    def gated_delta(self, y, state, proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta):
+        T = proj.shape[0]
+        scratch = torch.empty(T * (2 * sp.kv_heads * sp.dim + 2 * sp.heads * sp.vdim + 2 * sp.heads),
+                              device=proj.device, dtype=torch.float32)
+        self._delta.gated_delta(y, state[0], state[1], proj, conv_w, a_log, dt_bias, norm_w, meta.seq_cu, meta.seq_ctx,
+                              meta.seq_state, scratch, sp.heads, sp.kv_heads, sp.dim, sp.vdim, sp.conv, eps)
+
+    def delta_rule(self, out, state, proj, wl, a_b, w0, norm_w, sp, eps, meta, out_scale=1.0):
+        scratch = torch.empty(proj.shape[0] * 4 * sp.size, device=proj.device, dtype=torch.float32)
+        self._delta.delta_rule(out, state[0], proj, wl, a_b, w0, norm_w, meta.seq_cu, meta.seq_ctx, meta.seq_state,
+                             scratch, sp.heads, sp.dim, eps, out_scale)
+
+    ACTIVATIONS = {"tanh": 0, "xielu": 1}
+
+    def activation(self, out, x, kind, c0=0.0, c1=0.0):
+        self._delta.activation(out, x, self.ACTIVATIONS[kind], c0, c1)
+        return out
 
     def moe_align(self, experts, E, tile, slots, tile_expert, pair_slot):
         if E <= 128:
@@ -374,6 +463,24 @@ class ReferenceOps:
 
     def expert_gemm(self, out, x, w, slots, tile_expert, tile, gather_k, relu2):
         ref.expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2)
+
+    def attn_prepare(self, proj, cache, meta, inv_freq, sp, q_norm, k_norm, eps):
+        ref.attn_prepare(proj, cache, meta.positions, meta.slot_mapping, inv_freq, sp, q_norm, k_norm, eps)
+
+    def window_attention(self, out, proj, cache, meta, sp, gate_off, out_scale=1.0):
+        ref.window_attention(out, proj, cache, meta.seq_cu, meta.seq_ctx, meta.seq_bt, sp, gate_off, out_scale)
+
+    def gated_delta(self, y, state, proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta):
+        ref.gated_delta(y, state[0], state[1], proj, conv_w, a_log, dt_bias, norm_w, sp, eps, meta.seq_cu,
+                        meta.seq_ctx, meta.seq_state)
+
+    def delta_rule(self, out, state, proj, wl, a_b, w0, norm_w, sp, eps, meta, out_scale=1.0):
+        ref.delta_rule(out, state[0], proj, wl, a_b, w0, norm_w, sp, eps, meta.seq_cu, meta.seq_ctx,
+                       meta.seq_state, out_scale)
+
+    def activation(self, out, x, kind, c0=0.0, c1=0.0):
+        ref.activation(out, x, kind, c0, c1)
+        return out
 
     def sample(self, out_tok, out_lp, logits, temperature, top_k, top_p, seeds, steps, two_rounds=True):
         t, lp = ref.sample(logits, temperature, top_k, top_p, seeds, steps, bf16_row=False)

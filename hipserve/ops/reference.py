@@ -405,7 +405,7 @@ def scaled_add_group_rmsnorm(out, residual, w, groups, eps, mix=None, ls1=None, 
     out = residual normalised in ``groups`` equal consecutive parts, times w."""
     T, H = residual.shape
     if mix is not None:
-        residual += mix.float() * ls1.float()
+        residual += mix.float() * ls1.float() if ls1 is not None else mix.float()
     if y is not None:
         rows = y.float().index_select(0, pair_slot.long()).view(T, top, H)
         residual += rows.sum(1) * (1.0 / top) * ls2.float()
@@ -529,3 +529,162 @@ def expert_gemm(out, x, w, slots, tile_expert, tile, gather_k, relu2):
         if relu2:
             v = torch.relu(v) ** 2
         out[s] = v.to(out.dtype)
+
+
+# ---------------------------------------------------------------------------------
+# windowed sink attention on a paged [keys | values] cache, the two delta-rule
+# recurrences over state slots, per-head output norm + gate, elementwise activations
+
+def _rows_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def attn_prepare(proj, cache, positions, slots, inv_freq, sp, q_norm, k_norm, eps):
+    """proj rows = [q | k | v | ...] (after biases). In place on the q columns: the optional
+    whole-projection RMS norm (``sp.qk_norm``) and the rotation; the cache row of slots >= 0
+    gets [rotated keys | values], keys normed alike, values divided by their per-head root
+    mean square when ``sp.v_norm``."""
+    T = proj.shape[0]
+    nq, nk, nv = sp.q_size, sp.k_size, sp.v_size
+    p = proj.float()
+    q, k, v = p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:nq + nk + nv]
+    if sp.qk_norm:
+        q = _rows_rms(q, eps) * q_norm.float()
+        k = _rows_rms(k, eps) * k_norm.float()
+    q = partial_rope(q.reshape(T, sp.heads, sp.dim), positions, inv_freq).reshape(T, nq)
+    k = partial_rope(k.reshape(T, sp.kv_heads, sp.dim), positions, inv_freq).reshape(T, nk)
+    if sp.v_norm:
+        v = _rows_rms(v.reshape(T, sp.kv_heads, sp.vdim), eps).reshape(T, nv)
+    proj[:, :nq] = q.to(proj.dtype)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok]] = torch.cat([k, v], -1).to(cache.dtype)[ok]
+
+
+def window_attention(out, proj, cache, seq_cu, seq_ctx, seq_bt, sp, gate_off, out_scale):
+    """Per sequence s (rows cu[s]..cu[s+1]-1 at positions ctx[s]-n .. ctx[s]-1): head h scores
+    its prepared query against the cached keys of head h // (heads / kv_heads) with
+    0 <= pos - j < window; weights exp(s_j) / (sink + sum exp(s_j)); out[t, h * vdim ..] =
+    weighted values * sigmoid(proj[t, gate_off + h]) (gate_off >= 0) * out_scale."""
+    bs = cache.shape[1]
+    flat = cache.view(-1, cache.shape[-1])
+    cu = [int(x) for x in seq_cu]
+    H, G, d, dv, W = sp.heads, sp.kv_heads, sp.dim, sp.vdim, sp.window
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if a == b:
+            continue
+        ctx = int(seq_ctx[s])
+        pos = torch.arange(ctx - (b - a), ctx, device=proj.device)
+        lo = 0 if W <= 0 else max(0, int(pos[0]) - W + 1)
+        j = torch.arange(lo, ctx, device=proj.device)
+        kv = flat[seq_bt[s].long()[j // bs] * bs + j % bs].float()
+        k = kv[:, :G * d].view(-1, G, d).repeat_interleave(H // G, 1)
+        v = kv[:, G * d:].view(-1, G, dv).repeat_interleave(H // G, 1)
+        q = proj[a:b, :H * d].float().view(b - a, H, d)
+        sc = torch.einsum("nhd,jhd->hnj", q, k) * sp.scale
+        dd = pos[:, None] - j[None]
+        ok = (dd >= 0) & ((dd < W) if W > 0 else (dd >= 0))
+        sc = sc.masked_fill(~ok, float("-inf"))
+        m = sc.max(-1, keepdim=True).values
+        if sp.sink:
+            m = m.clamp(min=0.0)
+        e = torch.exp(sc - m)
+        den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sp.sink else 0.0)
+        o = torch.einsum("hnj,jhv->nhv", e / den, v)
+        if gate_off >= 0:
+            o = o * torch.sigmoid(proj[a:b, gate_off:gate_off + H].float()).unsqueeze(-1)
+        out[a:b] = (o * out_scale).reshape(b - a, H * dv).to(out.dtype)
+
+
+def _conv_inputs(proj, conv_state, a, b, start, slot, C, taps):
+    """The step's conv inputs of one sequence with the taps - 1 inputs before them in front."""
+    x = proj[a:b, :C].float()
+    prev = conv_state[slot][:taps - 1]
+    return torch.cat([prev if start > 0 else torch.zeros_like(prev), x], 0)
+
+
+def gated_delta(y, S, conv_state, proj, conv_w, a_log, dt_bias, norm_w, sp, eps, seq_cu, seq_ctx, seq_state):
+    """proj rows = [q | k | v | beta | decay | gate] pre-activations. Per sequence, from its slot
+    (zero when the step starts at position 0): causal conv + SiLU on q, k, v; unit q (times
+    dim^-1/2) and k; S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q; y = o / rms(o) *
+    norm_w * silu(gate). S [slots, heads, dim, vdim], conv_state [slots, taps - 1, channels]."""
+    H, G, d, dv, taps = sp.heads, sp.kv_heads, sp.dim, sp.vdim, sp.conv
+    C = sp.conv_channels
+    cu = [int(x) for x in seq_cu]
+    w = conv_w.float()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        n = b - a
+        if n == 0:
+            continue
+        slot, start = int(seq_state[s]), int(seq_ctx[s]) - n
+        xin = _conv_inputs(proj, conv_state, a, b, start, slot, C, taps)
+        xc = sum(xin[j:j + n] * w[:, j] for j in range(taps))
+        xc = xc * torch.sigmoid(xc)
+        if taps > 1:
+            conv_state[slot] = xin[n:]
+        q = xc[:, :G * d].view(n, G, d)
+        k = xc[:, G * d:2 * G * d].view(n, G, d)
+        v = xc[:, 2 * G * d:].view(n, H, dv)
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * d ** -0.5
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+        q, k = q.repeat_interleave(H // G, 1), k.repeat_interleave(H // G, 1)
+        p = proj[a:b, C:].float()
+        beta = torch.sigmoid(p[:, :H])
+        g = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(p[:, H:2 * H] + dt_bias.float()))
+        gate = p[:, 2 * H:].view(n, H, dv)
+        st = S[slot].clone() if start > 0 else torch.zeros_like(S[slot])
+        o = torch.empty(n, H, dv)
+        for t in range(n):
+            st = st * g[t, :, None, None]
+            u = beta[t, :, None] * (v[t] - torch.einsum("hkv,hk->hv", st, k[t]))
+            st = st + k[t, :, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hkv,hk->hv", st, q[t])
+        S[slot] = st
+        o = _rows_rms(o, eps) * norm_w.float() * (gate * torch.sigmoid(gate))
+        y[a:b] = o.reshape(n, H * dv).to(y.dtype)
+
+
+def delta_rule(out, S, proj, wl, a_b, w0, norm_w, sp, eps, seq_cu, seq_ctx, seq_state, out_scale):
+    """proj rows = [r | k | v | a | g | ...] pre-activations, wl the decay bottleneck's output
+    (fp32). Per head with u = unit(k): w = exp(-e^-1/2 sigmoid(wl + w0)), a = sigmoid(a + a_b),
+    S = diag(w) S - (a u)(u^T S) + k v^T (both terms on the old S), o = S^T r;
+    out = o / rms(o) * norm_w * sigmoid(g) * out_scale. S [slots, heads, dim(key), dim(value)]."""
+    H, d = sp.heads, sp.dim
+    N = H * d
+    cu = [int(x) for x in seq_cu]
+    for s in range(len(cu) - 1):
+        a0, b0 = cu[s], cu[s + 1]
+        n = b0 - a0
+        if n == 0:
+            continue
+        slot, start = int(seq_state[s]), int(seq_ctx[s]) - n
+        p = proj[a0:b0].float()
+        r, k, v = (p[:, i * N:(i + 1) * N].view(n, H, d) for i in range(3))
+        rem = torch.sigmoid(p[:, 3 * N:4 * N] + a_b.float()).view(n, H, d)
+        gate = torch.sigmoid(p[:, 4 * N:5 * N])
+        w = torch.exp(-0.6065306597126334 * torch.sigmoid(wl[a0:b0].float() + w0.float())).view(n, H, d)
+        u = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+        st = S[slot].clone() if start > 0 else torch.zeros_like(S[slot])
+        o = torch.empty(n, H, d)
+        for t in range(n):
+            uS = torch.einsum("hkv,hk->hv", st, u[t])
+            st = w[t, :, :, None] * st - (rem[t] * u[t])[:, :, None] * uS[:, None, :] + k[t, :, :, None] * v[t, :, None, :]
+            o[t] = torch.einsum("hkv,hk->hv", st, r[t])
+        S[slot] = st
+        o = _rows_rms(o, eps).reshape(n, N) * norm_w.float() * gate * out_scale
+        out[a0:b0] = o.to(out.dtype)
+
+
+def activation(out, x, kind, c0=0.0, c1=0.0):
+    """Elementwise: ``tanh``, or ``xielu`` with c0 = softplus(p), c1 = 1/2 + softplus(q):
+    c0 z^2 + z/2 for z > 0, c1 (exp(z) - 1 - z) + z/2 otherwise."""
+    z = x.float()
+    if kind == "tanh":
+        r = torch.tanh(z)
+    elif kind == "xielu":
+        zn = z.clamp(max=0.0)
+        r = torch.where(z > 0, c0 * z * z + 0.5 * z, c1 * (torch.expm1(zn) - zn) + 0.5 * z)
+    else:
+        raise ValueError(kind)
+    out.copy_(r.to(out.dtype))
