@@ -78,10 +78,10 @@ def parse():
     ap.add_argument("--tp-warmup", type=int, default=1)
     ap.add_argument("--tp-budget-s", type=float, default=150.0)
     ap.add_argument("--layer-compare", action="store_true",
-                    help="instead of the headline benchmark: prefill / decode tok/s of the Kesirax decoder "
-                         "beside a Mixtral-style model of equal size (hipserve/bench/layer_compare.py)")
+                    help="instead of the headline benchmark: prefill / decode tok/s of a layer-list decoder "
+                         "beside the closest family at equal size (hipserve/bench/layer_compare.py)")
     ap.add_argument("--layer-sizes", default="", help="with --layer-compare: sizes, comma separated (default: all)")
-    ap.add_argument("--layer-models", default="", help="with --layer-compare: kesirax, mixtral or both (default)")
+    ap.add_argument("--layer-models", default="", help="with --layer-compare: any of kesirax, mixtral, fikizen, dense (default: kesirax,mixtral)")
     ap.add_argument("--layer-batch", type=int, default=16)
     ap.add_argument("--layer-prompt", type=int, default=2048)
     ap.add_argument("--layer-new", type=int, default=64)

@@ -1,7 +1,9 @@
-"""``bench.py --layer-compare``: prefill and decode throughput of the Kesirax layer-list
-decoder at sizes that resemble a real model's layers, beside the closest existing family
-(Mixtral-style: sliding-window attention + MoE feed-forward) at equal size. Random-init
-weights, synthetic prompts, a few layers of each (the per-layer cost is what is compared).
+"""``bench.py --layer-compare``: prefill and decode throughput of the layer-list decoders at
+sizes that resemble a real model's layers, each beside the closest existing family at equal
+size: Kesirax beside a Mixtral-style model (sliding-window attention + MoE feed-forward),
+Fikizen beside a dense sliding-window model (grouped-query attention + gated dense
+feed-forward). Random-init weights, synthetic prompts, a few layers of each (the per-layer
+cost is what is compared). ``--layer-models`` picks the models; the ratios are given per pair.
 
 Per size and model, through the engine's own scheduler and step function:
   prefill tok/s  = batch x prompt_len / time of the steps that compute the prompts
@@ -15,9 +17,9 @@ import time
 
 SIZES = {
     # name: width, heads, window, experts, top, ff, gru width, vocab
-    "w1024": dict(width=1024, heads=8, window=512, experts=8, top=2, ff=512, gru=2048, vocab=32000),
-    "w2048": dict(width=2048, heads=16, window=1024, experts=16, top=2, ff=1024, gru=4096, vocab=32000),
-    "w4096": dict(width=4096, heads=32, window=1024, experts=8, top=2, ff=2048, gru=8192, vocab=32000),
+    "w1024": dict(width=1024, heads=8, window=512, experts=8, top=2, ff=512, gru=2048, vocab=32000, dense_ff=3072),
+    "w2048": dict(width=2048, heads=16, window=1024, experts=16, top=2, ff=1024, gru=4096, vocab=32000, dense_ff=6144),
+    "w4096": dict(width=4096, heads=32, window=1024, experts=8, top=2, ff=2048, gru=8192, vocab=32000, dense_ff=12288),
 }
 
 
@@ -40,6 +42,41 @@ def mixtral_config(name, s):
                        intermediate_size=s["ff"], vocab_size=s["vocab"], rope_theta=1e6,
                        max_position_embeddings=16384, num_experts=s["experts"], num_experts_per_tok=s["top"],
                        sliding_window=s["window"], layer_windows=(s["window"],) * 4, bos_token_id=1, eos_token_id=(2,))
+
+
+def fikizen_config(name, s):
+    """Four layers: gated sink attention + feed-forward, gated delta rule, attention beside the generalized
+    delta rule + feed-forward, the first layer's weights once more."""
+    from ..config import (DeltaRuleSpec, DenseFFSpec, FikizenConfig, GatedDeltaSpec, HybridLayerSpec,
+                          ParallelMixerSpec, WindowAttentionSpec)
+
+    H, kv = s["heads"], max(1, s["heads"] // 4)
+    attn = dict(heads=H, kv_heads=kv, dim=128, vdim=128, scale=128 ** -0.5, window=s["window"], rot_dims=64,
+                rot_base=5e5, sink=True)
+    a = WindowAttentionSpec(gate=True, **attn)
+    left = WindowAttentionSpec(bias=True, qk_norm=True, v_norm=True, **attn)
+    par = ParallelMixerSpec(left, DeltaRuleSpec(heads=s["width"] // 64, dim=64, decay_rank=64), 0.75, 1.25)
+    delta = GatedDeltaSpec(heads=H, kv_heads=kv, dim=128, vdim=128, conv=4)
+    f = DenseFFSpec(s["dense_ff"])
+    layers = (HybridLayerSpec(a, f), HybridLayerSpec(delta, None), HybridLayerSpec(par, f), HybridLayerSpec(a, f, 0))
+    return FikizenConfig(name=f"fikizen-{name}", hidden_size=s["width"], vocab_size=s["vocab"], layers=layers,
+                         logit_softcap=25.0, max_position_embeddings=16384, eos_token_id=(2,), bos_token_id=1)
+
+
+def dense_config(name, s):
+    """Four dense layers: sliding-window grouped-query attention + gated feed-forward whose three matrices
+    hold as many weights as the two of the design beside it (2/3 of its inner size)."""
+    from ..config import ModelConfig
+
+    return ModelConfig(name=f"dense-{name}", architecture="llama", family="llama", hidden_size=s["width"],
+                       num_layers=4, num_heads=s["heads"], num_kv_heads=max(1, s["heads"] // 4), head_dim=128,
+                       intermediate_size=s["dense_ff"] * 2 // 3 // 256 * 256, vocab_size=s["vocab"], rope_theta=1e6,
+                       max_position_embeddings=16384, sliding_window=s["window"], layer_windows=(s["window"],) * 4,
+                       bos_token_id=1, eos_token_id=(2,))
+
+
+MODELS = {"kesirax": kesirax_config, "mixtral": mixtral_config, "fikizen": fikizen_config, "dense": dense_config}
+PAIRS = (("kesirax", "mixtral"), ("fikizen", "dense"))
 
 
 def measure(mcfg, batch, prompt_len, new_tokens, device="cuda", repeats=2):
@@ -97,22 +134,23 @@ def main(args) -> int:
         s = SIZES[name]
         row = {"size": name, **s}
         models = [m for m in (args.layer_models or "kesirax,mixtral").split(",") if m]
-        for label, cfg in (("kesirax", kesirax_config(name, s)), ("mixtral", mixtral_config(name, s))):
-            if label not in models:
-                continue
+        for label in models:
+            cfg = MODELS[label](name, s)
             r = measure(cfg, args.layer_batch, args.layer_prompt, args.layer_new, device)
             row[label] = r
             print(json.dumps({"layer_compare": name, "model": cfg.name, "batch": args.layer_batch,
                               "prompt_len": args.layer_prompt, "new_tokens": args.layer_new, "dtype": "bf16",
                               "data": "synthetic", **r}), flush=True)
-        if "kesirax" not in row or "mixtral" not in row:
-            out.append(row)
-            continue
-        row["prefill_ratio"] = round(row["kesirax"]["prefill_tok_s"] / max(row["mixtral"]["prefill_tok_s"], 1e-9), 3)
-        row["decode_ratio"] = round(row["kesirax"]["decode_tok_s"] / max(row["mixtral"]["decode_tok_s"], 1e-9), 3)
+        for a, b in PAIRS:
+            if a in row and b in row:
+                row[f"{a}_vs_{b}"] = {k: round(row[a][f"{k}_tok_s"] / max(row[b][f"{k}_tok_s"], 1e-9), 3)
+                                      for k in ("prefill", "decode")}
+        if "kesirax_vs_mixtral" in row:
+            row["prefill_ratio"] = row["kesirax_vs_mixtral"]["prefill"]
+            row["decode_ratio"] = row["kesirax_vs_mixtral"]["decode"]
         out.append(row)
-    print(json.dumps({"layer_compare_summary": [{k: r.get(k) for k in ("size", "prefill_ratio", "decode_ratio")}
-                                                for r in out]}), flush=True)
+    keys = ("size", "prefill_ratio", "decode_ratio") + tuple(f"{a}_vs_{b}" for a, b in PAIRS)
+    print(json.dumps({"layer_compare_summary": [{k: r[k] for k in keys if k in r} for r in out]}), flush=True)
     if args.out:
         with open(args.out, "w") as f:
             json.dump(out, f, indent=1)
