@@ -81,7 +81,7 @@ void launch_window_attention_mfma(void* out, long out_ld, const void* proj, long
                                   hipStream_t s);
 
 // Delta-rule recurrences over state slots (delta_scan.hip). scratch: fp32, T * (2 * kv_heads * dim +
-// 2 * heads * vdim + 2 * heads) floats for the gated rule, T * 4 * heads * dim for the generalized one.
+// 2 * heads * vdim + 2 * heads) floats for the gated rule, T * 7 * heads * dim for the generalized one.
 int delta_max_dim();
 int delta_max_taps();
 void launch_gated_delta(void* y, float* S, float* conv_state, const void* proj, long ld, const float* conv_w,

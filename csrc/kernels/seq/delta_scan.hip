@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kScanThreads) void gated_delta_scan_kernel(
 }
 
 // proj rows = [r | k | v | a | g | ...] (N = heads * dim each), wl = decay pre-activation (fp32 [T, N]).
-// pre[t] = [w = exp(-e^-1/2 sigmoid(wl + w0)) | a u | u] with a = sigmoid(a + a_b), u = unit(k) per head.
+// pre[t] = [w = exp(-e^-1/2 sigmoid(wl + w0)) | a u | u | k | r | v] with a = sigmoid(a + a_b), u = unit(k) per head.
 template <typename T>
 __global__ __launch_bounds__(256) void delta_rule_prepare_kernel(
     float* __restrict__ pre, const T* __restrict__ proj, long ld, const float* __restrict__ wl,
@@ -238,9 +238,12 @@ __global__ __launch_bounds__(256) void delta_rule_prepare_kernel(
     for (int e = lane; e < dim; e += 64) {
       const int c = h * dim + e;
       const float u = ldf<T>(row, N + c) * inv;
-      pre[t * 3 * N + c] = expf(-0.60653065971263342f * sigmoid_f(wl[t * N + c] + w0[c]));
-      pre[t * 3 * N + N + c] = sigmoid_f(ldf<T>(row, 3 * N + c) + a_b[c]) * u;
-      pre[t * 3 * N + 2 * N + c] = u;
+      pre[t * 6 * N + c] = expf(-0.60653065971263342f * sigmoid_f(wl[t * N + c] + w0[c]));
+      pre[t * 6 * N + N + c] = sigmoid_f(ldf<T>(row, 3 * N + c) + a_b[c]) * u;
+      pre[t * 6 * N + 2 * N + c] = u;
+      pre[t * 6 * N + 3 * N + c] = ldf<T>(row, N + c);       // k, r, v as fp32: the scan reads one buffer
+      pre[t * 6 * N + 4 * N + c] = ldf<T>(row, c);
+      pre[t * 6 * N + 5 * N + c] = ldf<T>(row, 2 * N + c);
     }
   }
 }
@@ -251,7 +254,7 @@ __global__ __launch_bounds__(kScanThreads) void delta_rule_scan_kernel(
     const int* __restrict__ seq_cu, const int* __restrict__ seq_ctx, const int* __restrict__ seq_state, int heads,
     int dim) {
   constexpr int DP = kSeg * DS, TB = kTB;
-  __shared__ __attribute__((aligned(16))) float sv[TB][5][DP];  // w, a u, u, k, r (zero past dim)
+  __shared__ __attribute__((aligned(16))) float sv[TB][5][DP];  // w, a u, u, k, r (zero past dim), all from `pre`
   const int s = blockIdx.z, h = blockIdx.x, zb = blockIdx.y, tid = threadIdx.x;
   const int r0 = seq_cu[s], n = seq_cu[s + 1] - r0;
   if (n <= 0) return;
@@ -278,17 +281,14 @@ __global__ __launch_bounds__(kScanThreads) void delta_rule_scan_kernel(
       const long row = r0 + t0 + tt;
       const int c = h * dim + k;
       const bool in = tt < nt && k < dim;
-      rg[0][it] = in ? pre[row * 3 * N + c] : 0.f;
-      rg[1][it] = in ? pre[row * 3 * N + N + c] : 0.f;
-      rg[2][it] = in ? pre[row * 3 * N + 2 * N + c] : 0.f;
-      rg[3][it] = in ? ldf<T>(proj, row * ld + N + c) : 0.f;
-      rg[4][it] = in ? ldf<T>(proj, row * ld + c) : 0.f;
+#pragma unroll
+      for (int j = 0; j < 5; ++j) rg[j][it] = in ? pre[row * 6 * N + j * N + c] : 0.f;
     }
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt)
 #pragma unroll
       for (int cv = 0; cv < kCV; ++cv)
-        rv[tt][cv] = (tt < nt && v0 + cv < dim) ? ldf<T>(proj, (long)(r0 + t0 + tt) * ld + 2 * N + h * dim + v0 + cv) : 0.f;
+        rv[tt][cv] = (tt < nt && v0 + cv < dim) ? pre[(long)(r0 + t0 + tt) * 6 * N + 5 * N + h * dim + v0 + cv] : 0.f;
   };
   float* po = o + (long)r0 * N + h * dim + v0 + seg;
   fetch(0);
@@ -465,8 +465,8 @@ void launch_delta_rule(void* out, long out_ld, float* S, const void* proj, long 
                        float out_scale, bool f32, hipStream_t s) {
   if (nseq <= 0 || T <= 0) return;
   const int N = heads * dim;
-  float* pre = scratch;               // [T, 3 N]
-  float* o = pre + (long)T * 3 * N;   // [T, N]
+  float* pre = scratch;               // [T, 6 N]
+  float* o = pre + (long)T * 6 * N;   // [T, N]
   dim3 grid(heads, (dim + kCols - 1) / kCols, nseq);
   if (f32) {
     delta_rule_prepare_kernel<float><<<T, 256, 0, s>>>(pre, (const float*)proj, ld, wl, a_b, w0, heads, dim);

@@ -192,7 +192,7 @@ void delta_rule(at::Tensor& out, at::Tensor& S, const at::Tensor& proj, const at
   TORCH_CHECK(S.dim() == 4 && S.size(1) == heads && S.size(2) == dim && S.size(3) == dim);
   TORCH_CHECK(wl.numel() == T * N && a_b.numel() == N && w0.numel() == N && norm_w.numel() == N);
   TORCH_CHECK(seq_cu.numel() == nseq + 1 && seq_state.numel() >= nseq && nseq <= 65535 &&
-              scratch.numel() >= T * 4 * N);
+              scratch.numel() >= T * 7 * N);
   c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
   hipserve::launch_delta_rule(out.data_ptr(), out.stride(0), S.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
                               wl.data_ptr<float>(), a_b.data_ptr<float>(), w0.data_ptr<float>(),

@@ -320,7 +320,7 @@ class KernelOps:
                               meta.seq_state, scratch, sp.heads, sp.kv_heads, sp.dim, sp.vdim, sp.conv, eps)
 
     def delta_rule(self, out, state, proj, wl, a_b, w0, norm_w, sp, eps, meta, out_scale=1.0):
-        scratch = torch.empty(proj.shape[0] * 4 * sp.size, device=proj.device, dtype=torch.float32)
+        scratch = torch.empty(proj.shape[0] * 7 * sp.size, device=proj.device, dtype=torch.float32)
         self._delta.delta_rule(out, state[0], proj, wl, a_b, w0, norm_w, meta.seq_cu, meta.seq_ctx, meta.seq_state,
                              scratch, sp.heads, sp.dim, eps, out_scale)
 
