@@ -1,4 +1,4 @@
-// Window attention on the matrix cores (bf16 activations and cache), same contract as the generic
+// Window attention on the matrix cores (bf16 activations and cache), same interface as the generic
 // kernel of window_attention.hip: paged cache rows [all key heads | all value heads], sliding
 // window, optional softmax sink, optional per-head sigmoid output gate, output scale.
 //
