@@ -273,7 +273,7 @@ def _rope_params(d: dict, layer_type: str | None) -> tuple[float, dict | None]:
 _LLAMA3_SCALING = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                    "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
 
-# Public architecture hyper-parameters (SURVEY §2.E). Random-init weights of these
+# Public architecture hyper-parameters. Random-init weights of these
 # shapes are what the benchmarks run (no network => no checkpoints).
 PRESETS: dict[str, ModelConfig] = {
     "llama-3-8b": ModelConfig(name="llama-3-8b", hidden_size=4096, num_layers=32, num_heads=32,

@@ -376,7 +376,7 @@ def top_logprobs(logits, nreq, out_ids, out_lp):
 
     Exact over the whole row. The device kernel (csrc/kernels/penalties.hip
     top_logprobs) is exact too unless more than 64 keys share the bf16 bin of the n-th
-    largest value: it then keeps the lowest-index 64 of them (ADVICE r3), so in a row
+    largest value: it then keeps the lowest-index 64 of them, so in a row
     with > 64 logits within one bf16 ulp of the n-th largest the two may name different
     (equally probable to bf16 precision) entries."""
     K = out_ids.shape[1]
